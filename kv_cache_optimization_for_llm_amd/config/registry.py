@@ -68,6 +68,7 @@ NORMS = Registry("norm")
 POSITION_ENCODINGS = Registry("position encoding")
 BLOCKS = Registry("block arrangement")
 STREAM_OPS = Registry("operation between layers")
+LAYER_INPUTS = Registry("per-layer input")                 # what a layer adds to the stream from outside it (the token's own row of a table)
 ROTARY_FREQUENCIES = Registry("rotary frequency rule")     # name -> f(rot_dim, theta, **params) -> fp32 [rot_dim / 2]
 
 

@@ -1,7 +1,8 @@
 // Causal grouped-query attention over the paged cache: the plain kernel.
 //
 // One wavefront per (token, query head).  The query at absolute position p of its request
-// attends to keys lo..p of the same request (lo = 0, or p - window + 1 with a window), all read
+// attends to keys lo..p of the same request (lo = 0, or p - window + 1 with a window, or the start of
+// p's own chunk where positions see each other only inside chunks of a fixed size), all read
 // from the cache through the request's block-table row - the step has already written this
 // step's K and V there (the reference also scatters before it attends,
 // base/src/engine.cu:726-737).  Same recurrence as the reference's decode kernel
@@ -48,7 +49,7 @@ attention_rowwise_kernel(T *__restrict__ out, const T *__restrict__ q, int q_row
                          const int *__restrict__ block_table, int max_blocks,
                          const int *__restrict__ tok_seat, const int *__restrict__ tok_pos,
                          int num_q_heads, int num_kv_heads, int head_dim, int value_dim, int page_size,
-                         float scale, int window, int keep_first, const float *__restrict__ sinks) {
+                         float scale, int window, int keep_first, int chunk, const float *__restrict__ sinks) {
     __shared__ float q_s[ATTN_MAX_HEAD_DIM];
     __shared__ float p_s[KVA_WAVE];
     __shared__ long long voff_s[KVA_WAVE];
@@ -64,11 +65,11 @@ attention_rowwise_kernel(T *__restrict__ out, const T *__restrict__ q, int q_row
     for (int j = lane; j < head_dim; j += KVA_WAVE) q_s[j] = to_float(qrow[j]);
     __syncthreads();
 
-    const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    const int lo = kva_first_visible(pos, window, chunk);
     float m = -INFINITY, l = 0.f;
     float acc[ATTN_MAX_HEAD_DIM / KVA_WAVE] = {0.f, 0.f, 0.f, 0.f};
 
-    for (int kb = 0; kb <= pos / KVA_WAVE; ++kb) {
+    for (int kb = keep_first > 0 ? 0 : lo / KVA_WAVE; kb <= pos / KVA_WAVE; ++kb) {
         // a block with no visible key: behind the window and past the kept first positions
         if (kb * KVA_WAVE + KVA_WAVE <= lo && kb * KVA_WAVE >= keep_first) continue;
         const int key = kb * KVA_WAVE + lane;
@@ -135,7 +136,7 @@ extern "C" int kva_attention_rowwise(void *out, const void *q, int q_row_stride,
                                      const void *v_cache, const int *block_table, int max_blocks,
                                      const int *tok_seat, const int *tok_pos, int tokens,
                                      int num_q_heads, int num_kv_heads, int head_dim, int value_dim, int page_size,
-                                     float scale, int window, int keep_first, const float *sinks, int dtype,
+                                     float scale, int window, int keep_first, int chunk, const float *sinks, int dtype,
                                      hipStream_t stream) {
     KVA_REQUIRE(tokens >= 0 && num_q_heads > 0 && num_kv_heads > 0 && page_size > 0 && max_blocks > 0,
                 "attention: bad sizes");
@@ -146,7 +147,8 @@ extern "C" int kva_attention_rowwise(void *out, const void *q, int q_row_stride,
                 ATTN_MAX_HEAD_DIM);
     KVA_REQUIRE(q_row_stride % 4 == 0, "attention: query row stride %d must be a multiple of 4", q_row_stride);
     KVA_REQUIRE(num_q_heads <= 65535, "attention: too many heads");
-    KVA_REQUIRE(window >= 0 && keep_first >= 0, "attention: negative window or kept first positions");
+    KVA_REQUIRE(window >= 0 && keep_first >= 0 && chunk >= 0 && !(window > 0 && chunk > 0),
+                "attention: negative window, kept first positions or chunk, or a window together with chunks");
     KVA_REQUIRE(value_dim > 0 && value_dim <= ATTN_MAX_HEAD_DIM, "attention: value size %d must be at most %d",
                 value_dim, ATTN_MAX_HEAD_DIM);
     if (window == 0) keep_first = 0;
@@ -156,12 +158,12 @@ extern "C" int kva_attention_rowwise(void *out, const void *q, int q_row_stride,
         hipLaunchKernelGGL(attention_rowwise_kernel<float>, grid, block, 0, stream, (float *)out,
                            (const float *)q, q_row_stride, (const float *)k_cache,
                            (const float *)v_cache, block_table, max_blocks, tok_seat, tok_pos,
-                           num_q_heads, num_kv_heads, head_dim, value_dim, page_size, scale, window, keep_first, sinks);
+                           num_q_heads, num_kv_heads, head_dim, value_dim, page_size, scale, window, keep_first, chunk, sinks);
     else if (dtype == KVA_BF16)
         hipLaunchKernelGGL(attention_rowwise_kernel<bf16_t>, grid, block, 0, stream, (bf16_t *)out,
                            (const bf16_t *)q, q_row_stride, (const bf16_t *)k_cache,
                            (const bf16_t *)v_cache, block_table, max_blocks, tok_seat, tok_pos,
-                           num_q_heads, num_kv_heads, head_dim, value_dim, page_size, scale, window, keep_first, sinks);
+                           num_q_heads, num_kv_heads, head_dim, value_dim, page_size, scale, window, keep_first, chunk, sinks);
     else KVA_REQUIRE(false, "attention: unsupported dtype %d", dtype);
     KVA_CHECK_LAUNCH("attention_rowwise");
     return KVA_OK;

@@ -3,7 +3,8 @@
 //
 //  * kva_qk_encode_cache: heads of queries and keys whose first `rot` elements are rotated with
 //    either pairing (pair i = elements (i, i + rot/2) or (2i, 2i + 1)), optionally followed by a
-//    division of every head by its root mean square; keys of `head_dim` and values of another
+//    division of every head by its root mean square (and a multiplication by a weight per element,
+//    one for queries and one for keys: an RMS norm of every head); keys of `head_dim` and values of another
 //    size `value_dim` go to the paged K / V^T arrays (kv_layout.h).
 //  * kva_latent_encode_cache: a low-rank key/value entry.  Per token one latent vector of `rank`
 //    elements, RMS-normed with a weight, and one rotated key part of `rot` elements shared by all
@@ -24,7 +25,8 @@ qk_encode_cache_kernel(T *__restrict__ qkv, int row_stride, int k_off, int v_off
                        const float *__restrict__ sin_table, const int *__restrict__ positions,
                        const int *__restrict__ slot_mapping, int num_q_heads, int num_kv_heads, int head_dim,
                        int value_dim, int rot, int interleaved, float unit_eps, int page_size,
-                       const T *__restrict__ bias) {
+                       const T *__restrict__ bias, const float *__restrict__ q_weight,
+                       const float *__restrict__ k_weight) {
     const int t = blockIdx.x;
     const int lane = threadIdx.x % KVA_WAVE, wave = threadIdx.x / KVA_WAVE, waves = blockDim.x / KVA_WAVE;
     T *row = qkv + (size_t)t * row_stride;
@@ -75,6 +77,8 @@ qk_encode_cache_kernel(T *__restrict__ qkv, int row_stride, int k_off, int v_off
         }
         float mul = 1.f;
         if (unit_eps >= 0.f) mul = 1.0f / sqrtf(wave_sum(sq) / (float)head_dim + unit_eps);
+        // (optional) the weight of an RMS norm over the head, one per element, shared by the heads
+        const float *nw = is_q ? q_weight : k_weight;
         T *kdst = nullptr;
         const int kc = kva_k_chunk(head_dim);
         if (!is_q) kdst = k_cache + ((size_t)page * num_kv_heads + (head - num_q_heads)) * page_size * head_dim;
@@ -82,7 +86,7 @@ qk_encode_cache_kernel(T *__restrict__ qkv, int row_stride, int k_off, int v_off
         for (int c = 0; c < PER; ++c) {
             const int p = lane + c * KVA_WAVE;
             if (p >= pairs) continue;
-            const T r1 = from_float<T>(o1[c] * mul), r2 = from_float<T>(o2[c] * mul);
+            const T r1 = from_float<T>(o1[c] * mul * (nw ? nw[i1[c]] : 1.f)), r2 = from_float<T>(o2[c] * mul * (nw ? nw[i2[c]] : 1.f));
             if (is_q) {
                 h[i1[c]] = r1;
                 h[i2[c]] = r2;
@@ -176,8 +180,12 @@ extern "C" int kva_qk_encode_cache(void *qkv, int row_stride, int k_off, int v_o
                                    const float *cos_table, const float *sin_table, const int *positions,
                                    const int *slot_mapping, int tokens, int num_q_heads, int num_kv_heads,
                                    int head_dim, int value_dim, int rot, int interleaved, float unit_eps,
-                                   int page_size, int dtype, const void *bias, hipStream_t stream) {
-    KVA_REQUIRE(tokens >= 0 && num_q_heads > 0 && num_kv_heads > 0 && value_dim > 0, "qk_encode_cache: bad sizes");
+                                   int page_size, int dtype, const void *bias, const float *q_weight,
+                                   const float *k_weight, hipStream_t stream) {
+    // (num_kv_heads = 0: rows of queries alone, for a layer that reads another layer's keys and values)
+    KVA_REQUIRE(tokens >= 0 && num_q_heads > 0 && num_kv_heads >= 0 && value_dim > 0, "qk_encode_cache: bad sizes");
+    KVA_REQUIRE(num_kv_heads > 0 || !slot_mapping, "qk_encode_cache: a cache write without key heads");
+    KVA_REQUIRE((!q_weight && !k_weight) || unit_eps >= 0.f, "qk_encode_cache: a norm weight without the norm");
     KVA_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && head_dim <= ENC_MAX_HEAD_DIM,
                 "qk_encode_cache: head_dim %d must be even and at most %d", head_dim, ENC_MAX_HEAD_DIM);
     KVA_REQUIRE(rot >= 0 && rot <= head_dim && rot % 2 == 0,
@@ -191,7 +199,7 @@ extern "C" int kva_qk_encode_cache(void *qkv, int row_stride, int k_off, int v_o
     if (tokens == 0) return KVA_OK;
     if (rot == 0) cos_table = sin_table = reinterpret_cast<const float *>(qkv);     // never read
     const int vecs = head_dim / 8;
-    if (!bias && dtype == KVA_BF16 && interleaved && head_dim % 8 == 0 && (vecs & (vecs - 1)) == 0 && vecs <= KVA_WAVE &&
+    if (!bias && !q_weight && !k_weight && dtype == KVA_BF16 && interleaved && head_dim % 8 == 0 && (vecs & (vecs - 1)) == 0 && vecs <= KVA_WAVE &&
         row_stride % 8 == 0 && k_off % 8 == 0 && (reinterpret_cast<uintptr_t>(qkv) & 15) == 0) {
         hipLaunchKernelGGL(qk_encode_cache_vec_kernel, dim3(tokens), dim3(256), 0, stream, (bf16_t *)qkv, row_stride,
                            k_off, v_off, (bf16_t *)k_cache, (bf16_t *)v_cache, cos_table, sin_table, positions,
@@ -203,12 +211,12 @@ extern "C" int kva_qk_encode_cache(void *qkv, int row_stride, int k_off, int v_o
         hipLaunchKernelGGL(qk_encode_cache_kernel<float>, dim3(tokens), dim3(256), 0, stream, (float *)qkv, row_stride,
                            k_off, v_off, (float *)k_cache, (float *)v_cache, cos_table, sin_table, positions,
                            slot_mapping, num_q_heads, num_kv_heads, head_dim, value_dim, rot, interleaved, unit_eps,
-                           page_size, (const float *)bias);
+                           page_size, (const float *)bias, q_weight, k_weight);
     else if (dtype == KVA_BF16)
         hipLaunchKernelGGL(qk_encode_cache_kernel<bf16_t>, dim3(tokens), dim3(256), 0, stream, (bf16_t *)qkv,
                            row_stride, k_off, v_off, (bf16_t *)k_cache, (bf16_t *)v_cache, cos_table, sin_table,
                            positions, slot_mapping, num_q_heads, num_kv_heads, head_dim, value_dim, rot, interleaved,
-                           unit_eps, page_size, (const bf16_t *)bias);
+                           unit_eps, page_size, (const bf16_t *)bias, q_weight, k_weight);
     else KVA_REQUIRE(false, "qk_encode_cache: unsupported dtype %d", dtype);
     KVA_CHECK_LAUNCH("qk_encode_cache");
     return KVA_OK;

@@ -17,3 +17,11 @@ __host__ __device__ inline int kva_k_chunk(int head_dim) { return (head_dim & 7)
 __host__ __device__ inline size_t kva_k_at(int row, int dim, int page_size, int chunk) {
     return ((size_t)(dim / chunk) * page_size + row) * chunk + (dim % chunk);
 }
+
+// The first key a query at position `pos` sees: 0, or - with a window - the window's start
+// pos - window + 1, or - where positions see each other only inside chunks of `chunk` positions counted
+// from 0 - the start of the query's own chunk.  (Keys past `pos` are never seen.)
+__host__ __device__ inline int kva_first_visible(int pos, int window, int chunk) {
+    if (chunk > 0) return pos - pos % chunk;
+    return (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+}

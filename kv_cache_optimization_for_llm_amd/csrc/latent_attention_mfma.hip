@@ -19,6 +19,7 @@
 // term exp(sink) of its denominator) is added where the result is normalised.
 #include "common.h"
 #include "attention_frag.h"
+#include "kv_layout.h"
 #include <math.h>
 
 #define LAT_LOG2E 1.44269504088896340736f
@@ -308,7 +309,8 @@ extern "C" int kva_latent_attention_mfma(void *out, float *part_o, float *part_m
 // ---- grouped-query attention with the same options ---------------------------------------------
 //
 // The kernel above over the paged K / V^T arrays of ordinary attention (kv_layout.h), for what the
-// tuned kernels of attention_mfma.hip do not take: a window that keeps a request's first
+// tuned kernels of attention_mfma.hip do not take: chunks of positions that see only each other,
+// a window that keeps a request's first
 // positions visible, a sink per head, values of another size than the keys.  Rows of a tile are
 // (token, query head of the kv head's group) pairs, row = token_in_entry * G + head_in_group; one
 // wavefront per (item, kv head, key range).  D = 32 NKS key elements, DV = 16 NDT value elements.
@@ -320,8 +322,8 @@ gqa_attention_rows_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, 
                           const int *__restrict__ item_entry, const int *__restrict__ item_row0,
                           const int *__restrict__ entry_seat, const int *__restrict__ entry_q_start,
                           const int *__restrict__ entry_start_pos, int heads, int kv_heads, int page_size,
-                          float scale, int window, int keep_first, const float *__restrict__ sinks, int splits,
-                          int per_split) {
+                          float scale, int window, int keep_first, int chunk, const float *__restrict__ sinks,
+                          int splits, int per_split) {
     // RT tiles of 16 rows share every key and value fragment the wavefront loads (prompt portions:
     // half the loads a product with RT = 2)
     constexpr int DV = NDT * 16, D = NKS * 32;
@@ -337,8 +339,8 @@ gqa_attention_rows_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, 
     const int last_row = min(row0 + 16 * RT - 1, rows - 1);
     const int item_hi = start_pos + last_row / group;
     const int pos_lo = start_pos + row0 / group;
-    const int item_lo = (window > 0 && pos_lo - window + 1 > 0) ? pos_lo - window + 1 : 0;
-    const int hi_lo = (window > 0 && item_hi - window + 1 > 0) ? item_hi - window + 1 : 0;     // where the last row's window starts
+    const int item_lo = kva_first_visible(pos_lo, window, chunk);
+    const int hi_lo = kva_first_visible(item_hi, window, chunk);     // where the last row's window (or chunk) starts
     int my_pos[RT], my_lo[RT], my_head[RT];
     bool row_valid[RT];
     size_t my_token[RT];
@@ -351,7 +353,7 @@ gqa_attention_rows_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, 
         row_valid[rt] = row0 + 16 * rt + r < rows;
         my_pos[rt] = start_pos + row / group;
         my_head[rt] = kvh * group + row % group;
-        my_lo[rt] = (window > 0 && my_pos[rt] - window + 1 > 0) ? my_pos[rt] - window + 1 : 0;
+        my_lo[rt] = kva_first_visible(my_pos[rt], window, chunk);
         my_token[rt] = (size_t)q_start + row / group;
         const bf16_t *qrow = q + my_token[rt] * q_stride + (size_t)my_head[rt] * D + 8 * g;
 #pragma unroll
@@ -368,6 +370,7 @@ gqa_attention_rows_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, 
         k_begin = split * per_split;
         k_end = min(k_end, k_begin + per_split);
     }
+    if (keep_first == 0 && item_lo > k_begin) k_begin = min(item_lo & ~31, k_end);     // nothing in front is visible
     for (int kstart = k_begin & ~31; kstart < k_end; kstart += 32) {
         if (kstart + 32 <= item_lo && kstart >= keep_first) continue;
         int page[2];
@@ -513,7 +516,7 @@ extern "C" int kva_attention_rows_mfma(void *out, float *part_o, float *part_ml,
                                        const int *entry_seat, const int *entry_q_start, const int *entry_start_pos,
                                        int num_items, int total_rows, int heads, int kv_heads, int head_dim,
                                        int value_dim, int page_size, float scale, int window, int keep_first,
-                                       const float *sinks, int splits, int per_split, int row_tiles,
+                                       int chunk, const float *sinks, int splits, int per_split, int row_tiles,
                                        hipStream_t stream) {
     KVA_REQUIRE(kva_attention_rows_mfma_supported(head_dim, value_dim, page_size),
                 "attention_rows_mfma: no instance for keys of %d, values of %d, pages of %d", head_dim, value_dim, page_size);
@@ -523,7 +526,8 @@ extern "C" int kva_attention_rows_mfma(void *out, float *part_o, float *part_ml,
     KVA_REQUIRE(splits >= 1 && (long long)splits * kv_heads <= 65535 &&
                     (splits == 1 || (per_split > 0 && per_split % 32 == 0 && part_o && part_ml)),
                 "attention_rows_mfma: key ranges need a length that is a multiple of 32 and a workspace");
-    KVA_REQUIRE(window >= 0 && keep_first >= 0, "attention_rows_mfma: negative window or kept first positions");
+    KVA_REQUIRE(window >= 0 && keep_first >= 0 && chunk >= 0 && !(window > 0 && chunk > 0),
+                "attention_rows_mfma: negative window, kept first positions or chunk, or a window together with chunks");
     KVA_REQUIRE(row_tiles == 1 || (row_tiles == 2 && value_dim <= 128 && head_dim <= 128),
                 "attention_rows_mfma: one row tile an item, or two for heads up to 128");
     if (window == 0) keep_first = 0;
@@ -540,7 +544,7 @@ extern "C" int kva_attention_rows_mfma(void *out, float *part_o, float *part_ml,
                            part_ml, (const bf16_t *)q, q_stride, (const bf16_t *)k_cache,                        \
                            (const bf16_t *)v_cache, block_table, max_blocks, item_entry, item_row0, entry_seat,  \
                            entry_q_start, entry_start_pos, heads, kv_heads, page_size, scale, window,            \
-                           keep_first, sinks, splits, per_split);                                                \
+                           keep_first, chunk, sinks, splits, per_split);                                                \
         done = true;                                                                                             \
     }
     GQA_ROWS_INSTANCES(LAUNCH_ONE)

@@ -4,11 +4,13 @@
 //
 //  * kva_moe_route:  scores = softmax(logits) over all router outputs; the `top` largest of
 //    scores + correction are chosen; their weights are the plain scores (optionally renormalised).
+//    Or (`over_chosen`) the largest logits are chosen and the weights are the softmax over them alone.
 //  * kva_moe_align:  the (token, choice) slots of real experts sorted by expert into a list padded
 //    so that every tile of 16 rows belongs to one expert (`sorted_slot`, -1 = padding), with the
 //    expert of every tile (`tile_expert`, -1 = unused tile).
 //  * kva_moe_expert_rows: one product per tile against its expert's matrix.  Mode 0 ("up"): rows of
-//    x gathered by slot / top, activation applied, written at the sorted position.  Mode 1 ("down"):
+//    x gathered by slot / top, activation applied (a gated expert: act(gate) * up, its gate and up rows
+//    interleaved in one matrix), written at the sorted position.  Mode 1 ("down"):
 //    rows at the sorted position, times the slot's routing weight, written at the slot (fp32).
 //    bf16 with K % 32 == 0 runs on the matrix cores, everything else (fp32 too) on a plain tiled
 //    kernel that adds k ascending.
@@ -33,7 +35,8 @@ __device__ inline float moe_activate(float z, int act) {
 // ---- router ------------------------------------------------------------------------------
 __global__ void __launch_bounds__(256)
 moe_route_kernel(int *__restrict__ idx, float *__restrict__ wgt, const float *__restrict__ logits,
-                 const float *__restrict__ correction, int tokens, int outputs, int top, int renormalise) {
+                 const float *__restrict__ correction, int tokens, int outputs, int top, int renormalise,
+                 int over_chosen) {
     const int lane = threadIdx.x % KVA_WAVE;
     const int t = blockIdx.x * (blockDim.x / KVA_WAVE) + threadIdx.x / KVA_WAVE;
     if (t >= tokens) return;
@@ -57,8 +60,14 @@ moe_route_kernel(int *__restrict__ idx, float *__restrict__ wgt, const float *__
 #pragma unroll
     for (int j = 0; j < MOE_ROUTE_PER_LANE; ++j) {
         const int e = lane + j * KVA_WAVE;
-        s[j] = s[j] / sum;
-        ch[j] = e < outputs ? s[j] + (correction ? correction[e] : 0.f) : -INFINITY;
+        if (over_chosen) {
+            // the logits themselves are compared, and the weights are a softmax over the chosen ones
+            // alone: exp(logit - max) here, divided by the chosen ones' sum below
+            ch[j] = e < outputs ? logits[(size_t)t * outputs + e] + (correction ? correction[e] : 0.f) : -INFINITY;
+        } else {
+            s[j] = s[j] / sum;
+            ch[j] = e < outputs ? s[j] + (correction ? correction[e] : 0.f) : -INFINITY;
+        }
     }
     float total = 0.f;
     for (int k = 0; k < top; ++k) {
@@ -85,19 +94,19 @@ moe_route_kernel(int *__restrict__ idx, float *__restrict__ wgt, const float *__
             wgt[(size_t)t * top + k] = bs;
         }
     }
-    if (renormalise && lane == 0)
+    if ((renormalise || over_chosen) && lane == 0)
         for (int k = 0; k < top; ++k) wgt[(size_t)t * top + k] /= total;
 }
 
 extern "C" int kva_moe_route(int *idx, float *wgt, const float *logits, const float *correction, int tokens,
-                             int outputs, int top, int renormalise, hipStream_t stream) {
+                             int outputs, int top, int renormalise, int over_chosen, hipStream_t stream) {
     KVA_REQUIRE(idx && wgt && logits && tokens >= 0, "moe_route: missing operand");
     KVA_REQUIRE(outputs > 0 && outputs <= KVA_WAVE * MOE_ROUTE_PER_LANE, "moe_route: %d router outputs (at most %d)",
                 outputs, KVA_WAVE * MOE_ROUTE_PER_LANE);
     KVA_REQUIRE(top > 0 && top <= outputs, "moe_route: top %d of %d", top, outputs);
     if (tokens == 0) return KVA_OK;
     hipLaunchKernelGGL(moe_route_kernel, dim3((tokens + 3) / 4), dim3(256), 0, stream, idx, wgt, logits, correction,
-                       tokens, outputs, top, renormalise);
+                       tokens, outputs, top, renormalise, over_chosen);
     KVA_CHECK_LAUNCH("moe_route");
     return KVA_OK;
 }
@@ -151,7 +160,16 @@ struct MoeRows {
     const int *sorted_slot, *tile_expert;
     const float *slot_weight;       // mode 1
     int top, N, K, mode, act;
+    int gated;                      // mode 0: rows 2 j and 2 j + 1 of the matrix are output j's gate and up rows
 };
+
+// mode 0 of a gated expert: outputs n (even) and n + 1 of the product are one output of the layer
+__device__ inline void moe_store_gated(const MoeRows &a, void *out, int out_dtype, int place, int n, float gate, float up) {
+    const float v = moe_activate(gate, a.act) * up;
+    const size_t at = (size_t)place * (a.N / 2) + n / 2;
+    if (out_dtype == KVA_BF16) reinterpret_cast<uint16_t *>(out)[at] = float_to_bf16_bits(v);
+    else reinterpret_cast<float *>(out)[at] = v;
+}
 
 __device__ inline void moe_store(const MoeRows &a, void *out, int out_dtype, int place, int slot, int n, float v) {
     if (a.mode == 0) {
@@ -163,7 +181,7 @@ __device__ inline void moe_store(const MoeRows &a, void *out, int out_dtype, int
     }
 }
 
-// plain: a workgroup takes a tile of 16 rows and 64 outputs; thread (row, cx) 4 outputs
+// plain: a workgroup takes a tile of 16 rows and 64 outputs; thread (row, cx) 4 neighbouring outputs
 template <typename T>
 __global__ void __launch_bounds__(256)
 moe_expert_rows_kernel(MoeRows a, void *__restrict__ out, int out_dtype, const T *__restrict__ x,
@@ -191,13 +209,21 @@ moe_expert_rows_kernel(MoeRows a, void *__restrict__ out, int out_dtype, const T
         for (int kk = 0; kk < 32; ++kk) {
             const float xv = xs[row][kk];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[j] += xv * ws[cx + 16 * j][kk];
+            for (int j = 0; j < 4; ++j) acc[j] += xv * ws[4 * cx + j][kk];
         }
     }
     if (slot < 0) return;
+    if (a.gated) {
+#pragma unroll
+        for (int j = 0; j < 4; j += 2) {
+            const int n = n0 + 4 * cx + j;
+            if (n + 1 < a.N) moe_store_gated(a, out, out_dtype, place, n, acc[j], acc[j + 1]);
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const int n = n0 + cx + 16 * j;
+        const int n = n0 + 4 * cx + j;
         if (n < a.N) moe_store(a, out, out_dtype, place, slot, n, acc[j]);
     }
 }
@@ -263,14 +289,22 @@ __device__ inline void moe_tiles_product(const MoeRows &a, void *__restrict__ ou
     for (int rt = 0; rt < RT; ++rt) {
         if (slot[rt] < 0) continue;
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
+        for (int nt = 0; nt < NT; ++nt) {
+            float v[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int n = n_first + 16 * nt + 4 * g + i;
-                const float v = ((acc[nt][rt][i] + red[(0 * NT + nt) * RT + rt][lane][i]) + red[(1 * NT + nt) * RT + rt][lane][i])
-                                + red[(2 * NT + nt) * RT + rt][lane][i];
-                if (n < a.N) moe_store(a, out, out_dtype, place[rt], slot[rt], n, v);
+            for (int i = 0; i < 4; ++i)
+                v[i] = ((acc[nt][rt][i] + red[(0 * NT + nt) * RT + rt][lane][i]) + red[(1 * NT + nt) * RT + rt][lane][i])
+                       + red[(2 * NT + nt) * RT + rt][lane][i];
+            const int n = n_first + 16 * nt + 4 * g;
+            if (a.gated) {
+                if (n + 1 < a.N) moe_store_gated(a, out, out_dtype, place[rt], n, v[0], v[1]);
+                if (n + 3 < a.N) moe_store_gated(a, out, out_dtype, place[rt], n + 2, v[2], v[3]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (n + i < a.N) moe_store(a, out, out_dtype, place[rt], slot[rt], n + i, v[i]);
             }
+        }
     }
 }
 
@@ -296,7 +330,9 @@ moe_expert_rows_mfma_kernel(MoeRows a, void *__restrict__ out, int out_dtype, co
 
 extern "C" int kva_moe_expert_rows(void *out, int out_dtype, const void *x, const void *w, int dtype,
                                    const int *sorted_slot, const int *tile_expert, const float *slot_weight,
-                                   int max_tiles, int top, int N, int K, int mode, int act, hipStream_t stream) {
+                                   int max_tiles, int top, int N, int K, int mode, int act, int gated,
+                                   hipStream_t stream) {
+    KVA_REQUIRE(!gated || (mode == 0 && N % 2 == 0), "moe_expert_rows: gate and up rows come in pairs, in the first product");
     KVA_REQUIRE(out && x && w && sorted_slot && tile_expert, "moe_expert_rows: missing operand");
     KVA_REQUIRE(mode == 0 || (mode == 1 && slot_weight && out_dtype == KVA_F32),
                 "moe_expert_rows: mode 1 writes fp32 rows times a weight per slot");
@@ -304,7 +340,7 @@ extern "C" int kva_moe_expert_rows(void *out, int out_dtype, const void *x, cons
     KVA_REQUIRE(N > 0 && K > 0 && top > 0 && act >= 0 && act <= 3, "moe_expert_rows: bad sizes or activation");
     KVA_REQUIRE(max_tiles >= 0 && max_tiles <= 65535, "moe_expert_rows: %d tiles are too many for one launch", max_tiles);
     if (max_tiles == 0) return KVA_OK;
-    MoeRows a{sorted_slot, tile_expert, slot_weight, top, N, K, mode, act};
+    MoeRows a{sorted_slot, tile_expert, slot_weight, top, N, K, mode, act, gated};
     if (dtype == KVA_BF16 && K % 32 == 0) {
         // few tiles: 16 outputs a workgroup, so that enough of them stream the matrices; many: 64 outputs and
         // four row tiles, which share what they load
@@ -328,7 +364,8 @@ extern "C" int kva_moe_expert_rows(void *out, int out_dtype, const void *x, cons
 // ---- weighted sum --------------------------------------------------------------------------
 __global__ void __launch_bounds__(256)
 moe_combine_kernel(void *__restrict__ out, const void *__restrict__ x, int dtype, const float *__restrict__ rows,
-                   const int *__restrict__ idx, const float *__restrict__ wgt, int width, int top, int experts) {
+                   const int *__restrict__ idx, const float *__restrict__ wgt, const void *__restrict__ extra, int width,
+                   int top, int experts) {
     const size_t t = blockIdx.x;
     for (int j = threadIdx.x; j < width; j += blockDim.x) {
         float acc = 0.f;
@@ -338,18 +375,22 @@ moe_combine_kernel(void *__restrict__ out, const void *__restrict__ x, int dtype
             else acc += wgt[s] * (dtype == KVA_BF16 ? bf16_bits_to_float(reinterpret_cast<const uint16_t *>(x)[t * width + j])
                                                     : reinterpret_cast<const float *>(x)[t * width + j]);
         }
+        // what an expert that every token uses returned, with weight 1
+        if (extra) acc += dtype == KVA_BF16 ? bf16_bits_to_float(reinterpret_cast<const uint16_t *>(extra)[t * width + j])
+                                            : reinterpret_cast<const float *>(extra)[t * width + j];
         if (dtype == KVA_BF16) reinterpret_cast<uint16_t *>(out)[t * width + j] = float_to_bf16_bits(acc);
         else reinterpret_cast<float *>(out)[t * width + j] = acc;
     }
 }
 
 extern "C" int kva_moe_combine(void *out, const void *x, int dtype, const float *rows, const int *idx,
-                               const float *wgt, int tokens, int width, int top, int experts, hipStream_t stream) {
+                               const float *wgt, const void *extra, int tokens, int width, int top, int experts,
+                               hipStream_t stream) {
     KVA_REQUIRE(out && x && rows && idx && wgt && width > 0 && top > 0, "moe_combine: missing operand");
     KVA_REQUIRE(dtype == KVA_BF16 || dtype == KVA_F32, "moe_combine: unsupported dtype %d", dtype);
     if (tokens <= 0) return KVA_OK;
-    hipLaunchKernelGGL(moe_combine_kernel, dim3(tokens), dim3(256), 0, stream, out, x, dtype, rows, idx, wgt, width, top,
-                       experts);
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(tokens), dim3(256), 0, stream, out, x, dtype, rows, idx, wgt, extra, width,
+                       top, experts);
     KVA_CHECK_LAUNCH("moe_combine");
     return KVA_OK;
 }
@@ -388,8 +429,12 @@ __device__ inline void moe_ld8(const void *p, int dtype, size_t i, float (&f)[8]
 
 // the result as it is, plus a bias, or - with decay_inv_tau > 0 - turned into a decay:
 // sigmoid(z)^(1 / tau) = exp(-softplus(-z) / tau) with z = the sum plus its bias
-__device__ inline float small_product_finish(float acc, const float *bias, int n, float decay_inv_tau) {
+// or - with rate_log - into exp(-exp(rate_log[n / rate_group]) softplus(z)): a decay per output whose rate
+// is shared by groups of neighbouring outputs (the key channels of a head)
+__device__ inline float small_product_finish(float acc, const float *bias, int n, float decay_inv_tau,
+                                             const float *rate_log, int rate_group) {
     const float z = acc + (bias ? bias[n] : 0.f);
+    if (rate_log) return expf(-expf(rate_log[n / rate_group]) * (fmaxf(z, 0.f) + log1pf(expf(-fabsf(z)))));
     if (decay_inv_tau <= 0.f) return z;
     const float softplus = fmaxf(-z, 0.f) + log1pf(expf(-fabsf(z)));
     return expf(-softplus * decay_inv_tau);
@@ -398,7 +443,8 @@ __device__ inline float small_product_finish(float acc, const float *bias, int n
 __global__ void __launch_bounds__(256)
 small_product_f32_kernel(float *__restrict__ out, const void *__restrict__ x, int x_dtype, int x_stride,
                          const void *__restrict__ w, int w_dtype, int N, int K, int per_block,
-                         const float *__restrict__ bias, float decay_inv_tau) {
+                         const float *__restrict__ bias, float decay_inv_tau, const float *__restrict__ rate_log,
+                         int rate_group) {
     extern __shared__ float xs[];
     const size_t t = blockIdx.x;
     const int n_lo = blockIdx.y * per_block, n_hi = min(N, n_lo + per_block);
@@ -417,7 +463,7 @@ small_product_f32_kernel(float *__restrict__ out, const void *__restrict__ x, in
             }
             for (int k = K8 + lane; k < K; k += KVA_WAVE) acc += xs[k] * moe_ld(w, w_dtype, (size_t)n * K + k);
             acc = wave_sum(acc);
-            if (lane == 0) out[t * N + n] = small_product_finish(acc, bias, n, decay_inv_tau);
+            if (lane == 0) out[t * N + n] = small_product_finish(acc, bias, n, decay_inv_tau, rate_log, rate_group);
         }
     } else {
         for (int n = n_lo + threadIdx.x; n < n_hi; n += blockDim.x) {
@@ -429,14 +475,16 @@ small_product_f32_kernel(float *__restrict__ out, const void *__restrict__ x, in
                 for (int i = 0; i < 8; ++i) acc += xs[k + i] * f[i];
             }
             for (int k = K8; k < K; ++k) acc += xs[k] * moe_ld(w, w_dtype, (size_t)n * K + k);
-            out[t * N + n] = small_product_finish(acc, bias, n, decay_inv_tau);
+            out[t * N + n] = small_product_finish(acc, bias, n, decay_inv_tau, rate_log, rate_group);
         }
     }
 }
 
 extern "C" int kva_small_product_f32(float *out, const void *x, int x_dtype, int x_stride, const void *w, int w_dtype,
                                      int tokens, int N, int K, const float *bias, float decay_inv_tau,
-                                     hipStream_t stream) {
+                                     const float *rate_log, int rate_group, hipStream_t stream) {
+    KVA_REQUIRE(!rate_log || (rate_group > 0 && N % rate_group == 0 && decay_inv_tau <= 0.f),
+                "small_product_f32: rates are shared by whole groups of outputs, and exclude the other decay");
     KVA_REQUIRE(out && x && w && tokens >= 0 && N > 0, "small_product_f32: missing operand or bad sizes");
     KVA_REQUIRE(K > 0 && K <= SMALL_PRODUCT_MAX_K && x_stride >= K, "small_product_f32: K %d must lie in 1..%d", K, SMALL_PRODUCT_MAX_K);
     KVA_REQUIRE((x_dtype == KVA_BF16 || x_dtype == KVA_F32) && (w_dtype == KVA_BF16 || w_dtype == KVA_F32),
@@ -447,7 +495,8 @@ extern "C" int kva_small_product_f32(float *out, const void *x, int x_dtype, int
     const int blocks_y = (N + per_block - 1) / per_block;
     KVA_REQUIRE(tokens <= 0x7fffffff && blocks_y <= 65535, "small_product_f32: too many outputs");
     hipLaunchKernelGGL(small_product_f32_kernel, dim3(tokens, blocks_y), dim3(256), (size_t)K * sizeof(float), stream,
-                       out, x, x_dtype, x_stride, w, w_dtype, N, K, per_block, bias, decay_inv_tau);
+                       out, x, x_dtype, x_stride, w, w_dtype, N, K, per_block, bias, decay_inv_tau, rate_log,
+                       rate_group > 0 ? rate_group : 1);
     KVA_CHECK_LAUNCH("small_product_f32");
     return KVA_OK;
 }

@@ -3,9 +3,11 @@
 //  * kva_causal_conv_act / kva_conv_state_update: a short causal convolution over time per channel
 //    followed by silu; the last taps - 1 inputs of a request are part of its state.
 //  * kva_gated_delta_rule: per head S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q with
-//    unit-norm q and k, one decay g = exp(-exp(A_log) softplus(a + dt_bias)) per head and token.
+//    unit-norm q and k, one decay g = exp(-exp(A_log) softplus(a + dt_bias)) per head and token - or a
+//    decay per head and key channel, handed in ready-made, that multiplies the rows of S one by one.
 //  * kva_gated_linear_attention: per head S <- diag(alpha) S + k v^T; o = S^T q with a decay per
-//    key channel, alpha = sigmoid(z)^(1 / tau).
+//    key channel, alpha = sigmoid(z)^(1 / tau) - or one fixed decay a head for all channels and tokens;
+//    q, k and v may pass an activation (silu) on their way in.
 //  * kva_head_norm_gate: every head of a row divided by its root mean square (optional) times a
 //    weight, times act(gate), times a constant, into a column range of a wider buffer.
 //
@@ -36,6 +38,7 @@ __device__ inline void rec_st(void *p, int dtype, size_t i, float v) {
 __device__ inline float rec_sigmoid(float z) { return 1.f / (1.f + expf(-z)); }
 __device__ inline float rec_silu(float z) { return z / (1.f + expf(-z)); }
 __device__ inline float rec_softplus(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
+__device__ inline float rec_act(float z, int act) { return act == 1 ? rec_silu(z) : z; }
 
 // sum over the lanes that share a column (lanes c, c + 16, c + 32, c + 48), all of them get it
 __device__ inline float rec_column_sum(float v) {
@@ -130,7 +133,8 @@ struct RecArgs {
 __global__ void __launch_bounds__(KVA_WAVE)
 gated_delta_rule_kernel(RecArgs a, const float *__restrict__ qkv, int conv_stride, const void *__restrict__ y,
                         int y_dtype, int y_stride, int beta_off, int decay_off, const float *__restrict__ a_log,
-                        const float *__restrict__ dt_bias, float unit_eps) {
+                        const float *__restrict__ dt_bias, float unit_eps, const float *__restrict__ channel_decay,
+                        int decay_stride) {
     extern __shared__ float lds[];
     const int lane = threadIdx.x, c = lane % REC_COLS, r = lane / REC_COLS;
     const int slices = (a.vdim + REC_COLS - 1) / REC_COLS;
@@ -141,10 +145,12 @@ gated_delta_rule_kernel(RecArgs a, const float *__restrict__ qkv, int conv_strid
     const int d = a.dim, dv = a.vdim, kvh = head / (a.heads / a.kv_heads);
     const bool on = col < dv;
     float *S = lds, *qs = S + d * REC_COLS, *ks = qs + a.chunk * d, *bs = ks + a.chunk * d, *gs = bs + a.chunk;
+    float *as = gs + a.chunk;            // with a decay per key channel: the chunk's decays [chunk][dim]
     float *Sg = a.state + (size_t)a.entry_seat[e] * a.seat_stride + a.state_off + (size_t)head * d * dv;
     for (int i = r; i < d; i += REC_ROWGROUPS) S[i * REC_COLS + c] = on ? Sg[(size_t)i * dv + col] : 0.f;
     const int k_col = a.kv_heads * d, v_col = 2 * a.kv_heads * d;
-    const float rate = expf(a_log[head]), bias = dt_bias[head], q_mul = 1.0f / sqrtf((float)d);
+    const float rate = channel_decay ? 0.f : expf(a_log[head]), bias = channel_decay ? 0.f : dt_bias[head];
+    const float q_mul = 1.0f / sqrtf((float)d);
     for (int t0 = 0; t0 < n; t0 += a.chunk) {
         const int m = min(a.chunk, n - t0);
         __syncthreads();
@@ -152,6 +158,7 @@ gated_delta_rule_kernel(RecArgs a, const float *__restrict__ qkv, int conv_strid
             const size_t row = (size_t)(q0 + t0 + x / d) * conv_stride;
             qs[x] = qkv[row + kvh * d + x % d];
             ks[x] = qkv[row + k_col + kvh * d + x % d];
+            if (channel_decay) as[x] = channel_decay[(size_t)(q0 + t0 + x / d) * decay_stride + head * d + x % d];
         }
         __syncthreads();
         // unit vectors: token tt by the four lanes 4 tt .. 4 tt + 3 (chunk <= 16)
@@ -175,7 +182,7 @@ gated_delta_rule_kernel(RecArgs a, const float *__restrict__ qkv, int conv_strid
                 if (part == 0) {
                     const size_t yrow = (size_t)(q0 + t0 + tt) * y_stride;
                     bs[tt] = rec_sigmoid(rec_ld(y, y_dtype, yrow + beta_off + head));
-                    gs[tt] = expf(-rate * rec_softplus(rec_ld(y, y_dtype, yrow + decay_off + head) + bias));
+                    gs[tt] = channel_decay ? 1.f : expf(-rate * rec_softplus(rec_ld(y, y_dtype, yrow + decay_off + head) + bias));
                 }
             }
         }
@@ -186,6 +193,10 @@ gated_delta_rule_kernel(RecArgs a, const float *__restrict__ qkv, int conv_strid
             const size_t row = (size_t)(q0 + t0 + tt);
             const float v = on ? qkv[row * conv_stride + v_col + head * dv + col] : 0.f;
             float dot = 0.f;
+            if (channel_decay) {      // the rows of S are decayed one by one before S^T k is taken
+                const float *al = as + tt * d;
+                for (int i = r; i < d; i += REC_ROWGROUPS) S[i * REC_COLS + c] *= al[i];
+            }
             for (int i = r; i < d; i += REC_ROWGROUPS) dot += S[i * REC_COLS + c] * k[i];
             dot = rec_column_sum(dot);
             const float u = beta * (v - g * dot);
@@ -207,7 +218,8 @@ gated_delta_rule_kernel(RecArgs a, const float *__restrict__ qkv, int conv_strid
 // decays alpha (heads x dim a token, fp32) come in a buffer of their own; q is multiplied by q_mul.
 __global__ void __launch_bounds__(KVA_WAVE)
 gated_linear_attention_kernel(RecArgs a, const void *__restrict__ y, int y_dtype, int y_stride, int q_off, int k_off,
-                              int v_off, const float *__restrict__ alpha, int alpha_stride, float q_mul) {
+                              int v_off, const float *__restrict__ alpha, int alpha_stride, float q_mul,
+                              const float *__restrict__ head_decay, int act) {
     extern __shared__ float lds[];
     const int lane = threadIdx.x, c = lane % REC_COLS, r = lane / REC_COLS;
     const int slices = (a.vdim + REC_COLS - 1) / REC_COLS;
@@ -226,15 +238,15 @@ gated_linear_attention_kernel(RecArgs a, const void *__restrict__ y, int y_dtype
         for (int x = lane; x < m * d; x += KVA_WAVE) {
             const size_t row = (size_t)(q0 + t0 + x / d);
             const int i = head * d + x % d;
-            qs[x] = rec_ld(y, y_dtype, row * y_stride + q_off + i) * q_mul;
-            ks[x] = rec_ld(y, y_dtype, row * y_stride + k_off + i);
-            as[x] = alpha[row * alpha_stride + i];
+            qs[x] = rec_act(rec_ld(y, y_dtype, row * y_stride + q_off + i), act) * q_mul;
+            ks[x] = rec_act(rec_ld(y, y_dtype, row * y_stride + k_off + i), act);
+            as[x] = alpha ? alpha[row * alpha_stride + i] : head_decay[head];
         }
         __syncthreads();
         for (int tt = 0; tt < m; ++tt) {
             const float *q = qs + tt * d, *k = ks + tt * d, *al = as + tt * d;
             const size_t row = (size_t)(q0 + t0 + tt);
-            const float v = on ? rec_ld(y, y_dtype, row * y_stride + v_off + head * dv + col) : 0.f;
+            const float v = on ? rec_act(rec_ld(y, y_dtype, row * y_stride + v_off + head * dv + col), act) : 0.f;
             float o = 0.f;
             for (int i = r; i < d; i += REC_ROWGROUPS) {
                 const float s = al[i] * S[i * REC_COLS + c] + k[i] * v;
@@ -289,14 +301,18 @@ __device__ inline void row16_sum_each(float (&x)[N]) {
     for (int i = 0; i < N; ++i) x[i] += t[i];
 }
 
-template <int RP>
+// CD: the decay has one value per head and key channel and comes ready-made, fp32 [T, heads * dim]
+// (`channel_decay`); the rows of S are then decayed one by one and the head's single decay is not formed.
+template <int RP, bool CD>
 __global__ void __launch_bounds__(REG_THREADS)
 gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_stride, const void *__restrict__ y,
                             int y_dtype, int y_stride, int beta_off, int decay_off, const float *__restrict__ a_log,
-                            const float *__restrict__ dt_bias, float unit_eps) {
+                            const float *__restrict__ dt_bias, float unit_eps, const float *__restrict__ channel_decay,
+                            int decay_stride) {
     constexpr int DP = REG_LANES * RP, DS = DP + 4, CH = REC_CHUNK, PER = CH * DP / REG_THREADS;   // token rows 4 banks apart
     __shared__ __attribute__((aligned(16))) float qs[CH * DS];
     __shared__ __attribute__((aligned(16))) float ks[CH * DS];
+    __shared__ __attribute__((aligned(16))) float as[CD ? CH * DS : 4];
     __shared__ float vs[CH * REG_BLOCK_COLS], os[CH * REG_BLOCK_COLS], bs[CH], gs[CH], nq[CH], nk[CH];
     const int tid = threadIdx.x, lane = tid % KVA_WAVE, wave = tid / KVA_WAVE;
     const int c = lane / REG_LANES, r = lane % REG_LANES;
@@ -316,19 +332,21 @@ gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_s
         S[j] = (on && i < d) ? Sg[(size_t)i * dv + col] : 0.f;
     }
     const int k_col = a.kv_heads * d, v_col = 2 * a.kv_heads * d;
-    const float rate = expf(a_log[head]), bias = dt_bias[head], q_mul = 1.0f / sqrtf((float)d);
+    const float rate = CD ? 0.f : expf(a_log[head]), bias = CD ? 0.f : dt_bias[head], q_mul = 1.0f / sqrtf((float)d);
     constexpr int VPER = CH * REG_BLOCK_COLS / REG_THREADS;
-    float pq[PER], pk[PER], pv[VPER], pb = 0.f, pg = 0.f;
+    float pq[PER], pk[PER], pa[CD ? PER : 1], pv[VPER], pb = 0.f, pg = 0.f;
     auto fetch = [&](int t0, int m) {
 #pragma unroll
         for (int j = 0; j < PER; ++j) {
             pq[j] = pk[j] = 0.f;
+            if constexpr (CD) pa[j] = 0.f;
             if (REG_THREADS * j / DP >= m) continue;        // (the whole workgroup: a decoded token loads one row)
             const int x = tid + REG_THREADS * j, tt = x / DP, i = x % DP;
             if (tt >= m || i >= d) continue;
             const size_t row = (size_t)(q0 + t0 + tt) * conv_stride;
             pq[j] = qkv[row + kvh * d + i];
             pk[j] = qkv[row + k_col + kvh * d + i];
+            if constexpr (CD) pa[j] = channel_decay[(size_t)(q0 + t0 + tt) * decay_stride + head * d + i];
         }
 #pragma unroll
         for (int j = 0; j < VPER; ++j) {   // the chunk's tokens x 16 columns
@@ -339,7 +357,7 @@ gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_s
         if (tid < m) {
             const size_t yrow = (size_t)(q0 + t0 + tid) * y_stride;
             pb = rec_ld(y, y_dtype, yrow + beta_off + head);
-            pg = rec_ld(y, y_dtype, yrow + decay_off + head);
+            if constexpr (!CD) pg = rec_ld(y, y_dtype, yrow + decay_off + head);
         }
     };
     fetch(0, min(CH, n));
@@ -351,12 +369,13 @@ gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_s
             const int x = tid + REG_THREADS * j, at = (x / DP) * DS + x % DP;
             qs[at] = pq[j];
             ks[at] = pk[j];
+            if constexpr (CD) as[at] = pa[j];
         }
 #pragma unroll
         for (int j = 0; j < VPER; ++j) vs[tid + REG_THREADS * j] = pv[j];
         if (tid < m) {
             bs[tid] = rec_sigmoid(pb);
-            gs[tid] = expf(-rate * rec_softplus(pg + bias));
+            gs[tid] = CD ? 1.f : expf(-rate * rec_softplus(pg + bias));
         }
         __syncthreads();
         if (wave < CH / 16) {   // what makes q and k unit vectors: a token by four lanes, every fourth element each
@@ -391,6 +410,7 @@ gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_s
             const float4 *q4 = reinterpret_cast<const float4 *>(qs + at * DS) + r;
             const float g = gs[at], beta = bs[at], v = vs[at * REG_BLOCK_COLS + wave * REG_COLS + c], mq = nq[at], mk = nk[at];
             float4 kk[RP / 4], qq[RP / 4];
+            float Sd[CD ? RP : 1];               // the decayed rows, where every row has a decay of its own
             float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f, p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;
 #pragma unroll
             for (int j = 0; j < RP / 4; ++j) {
@@ -398,13 +418,25 @@ gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_s
                 qq[j] = q4[REG_LANES * j];
                 // the unit vectors' factors multiply the sums: S^T (mk k) = mk (S^T k), S^T (mq q) likewise
                 kk[j].x *= mk; kk[j].y *= mk; kk[j].z *= mk; kk[j].w *= mk;
-                d0 += S[4 * j] * kk[j].x;
+                if constexpr (CD) {
+                    const float4 al = (reinterpret_cast<const float4 *>(as + at * DS) + r)[REG_LANES * j];
+                    Sd[4 * j] = al.x * S[4 * j];
+                    Sd[4 * j + 1] = al.y * S[4 * j + 1];
+                    Sd[4 * j + 2] = al.z * S[4 * j + 2];
+                    Sd[4 * j + 3] = al.w * S[4 * j + 3];
+                    d0 += Sd[4 * j] * kk[j].x;
+                    d1 += Sd[4 * j + 1] * kk[j].y;
+                    d2 += Sd[4 * j + 2] * kk[j].z;
+                    d3 += Sd[4 * j + 3] * kk[j].w;
+                } else {
+                    d0 += S[4 * j] * kk[j].x;
+                    d1 += S[4 * j + 1] * kk[j].y;
+                    d2 += S[4 * j + 2] * kk[j].z;
+                    d3 += S[4 * j + 3] * kk[j].w;
+                }
                 p0 += S[4 * j] * qp[j].x;
-                d1 += S[4 * j + 1] * kk[j].y;
                 p1 += S[4 * j + 1] * qp[j].y;
-                d2 += S[4 * j + 2] * kk[j].z;
                 p2 += S[4 * j + 2] * qp[j].z;
-                d3 += S[4 * j + 3] * kk[j].w;
                 p3 += S[4 * j + 3] * qp[j].w;
             }
             d0 += d1; p0 += p1; d2 += d3; p2 += p3;
@@ -415,10 +447,17 @@ gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_s
             const float u = beta * (v - g * both[0]);
 #pragma unroll
             for (int j = 0; j < RP / 4; ++j) {
-                S[4 * j] = g * S[4 * j] + kk[j].x * u;
-                S[4 * j + 1] = g * S[4 * j + 1] + kk[j].y * u;
-                S[4 * j + 2] = g * S[4 * j + 2] + kk[j].z * u;
-                S[4 * j + 3] = g * S[4 * j + 3] + kk[j].w * u;
+                if constexpr (CD) {
+                    S[4 * j] = Sd[4 * j] + kk[j].x * u;
+                    S[4 * j + 1] = Sd[4 * j + 1] + kk[j].y * u;
+                    S[4 * j + 2] = Sd[4 * j + 2] + kk[j].z * u;
+                    S[4 * j + 3] = Sd[4 * j + 3] + kk[j].w * u;
+                } else {
+                    S[4 * j] = g * S[4 * j] + kk[j].x * u;
+                    S[4 * j + 1] = g * S[4 * j + 1] + kk[j].y * u;
+                    S[4 * j + 2] = g * S[4 * j + 2] + kk[j].z * u;
+                    S[4 * j + 3] = g * S[4 * j + 3] + kk[j].w * u;
+                }
                 qp[j] = qq[j];
             }
             mqp = mq;
@@ -443,7 +482,8 @@ gated_delta_rule_reg_kernel(RecArgs a, const float *__restrict__ qkv, int conv_s
 template <int RP>
 __global__ void __launch_bounds__(REG_THREADS)
 gated_linear_attention_reg_kernel(RecArgs a, const void *__restrict__ y, int y_dtype, int y_stride, int q_off, int k_off,
-                                  int v_off, const float *__restrict__ alpha, int alpha_stride, float q_mul) {
+                                  int v_off, const float *__restrict__ alpha, int alpha_stride, float q_mul,
+                                  const float *__restrict__ head_decay, int act) {
     constexpr int DP = REG_LANES * RP, DS = DP + 4, CH = REC_CHUNK, PER = CH * DP / REG_THREADS;   // token rows 4 banks apart
     __shared__ __attribute__((aligned(16))) float qs[CH * DS];
     __shared__ __attribute__((aligned(16))) float ks[CH * DS];
@@ -468,6 +508,7 @@ gated_linear_attention_reg_kernel(RecArgs a, const void *__restrict__ y, int y_d
     }
     constexpr int VPER = CH * REG_BLOCK_COLS / REG_THREADS;
     float pq[PER], pk[PER], pa[PER], pv[VPER];
+    const float fixed = alpha ? 0.f : head_decay[head];     // one decay for the head's every channel and token
     auto fetch = [&](int t0, int m) {
 #pragma unroll
         for (int j = 0; j < PER; ++j) {
@@ -476,15 +517,15 @@ gated_linear_attention_reg_kernel(RecArgs a, const void *__restrict__ y, int y_d
             const int x = tid + REG_THREADS * j, tt = x / DP, i = x % DP;
             if (tt >= m || i >= d) continue;
             const size_t row = (size_t)(q0 + t0 + tt);
-            pq[j] = rec_ld(y, y_dtype, row * y_stride + q_off + head * d + i);
-            pk[j] = rec_ld(y, y_dtype, row * y_stride + k_off + head * d + i);
-            pa[j] = alpha[row * alpha_stride + head * d + i];
+            pq[j] = rec_act(rec_ld(y, y_dtype, row * y_stride + q_off + head * d + i), act);
+            pk[j] = rec_act(rec_ld(y, y_dtype, row * y_stride + k_off + head * d + i), act);
+            pa[j] = alpha ? alpha[row * alpha_stride + head * d + i] : fixed;
         }
 #pragma unroll
         for (int j = 0; j < VPER; ++j) {   // the chunk's tokens x 16 columns
             const int x = tid + REG_THREADS * j, tt = x / REG_BLOCK_COLS, cc = x % REG_BLOCK_COLS;
             pv[j] = (tt < m && block_col0 + cc < dv)
-                        ? rec_ld(y, y_dtype, (size_t)(q0 + t0 + tt) * y_stride + v_off + head * dv + block_col0 + cc) : 0.f;
+                        ? rec_act(rec_ld(y, y_dtype, (size_t)(q0 + t0 + tt) * y_stride + v_off + head * dv + block_col0 + cc), act) : 0.f;
         }
     };
     fetch(0, min(CH, n));
@@ -581,30 +622,44 @@ static int rec_check(const char *what, const void *out, const void *state, const
 extern "C" int kva_gated_delta_rule(float *out, float *state, long long seat_stride, int state_off, const float *qkv,
                                     int conv_stride, const void *y, int y_dtype, int y_stride, int beta_off,
                                     int decay_off, const float *a_log, const float *dt_bias, float unit_eps,
+                                    const float *channel_decay, int decay_stride,
                                     const int *entry_q_start, const int *entry_seat, int entries, int heads,
                                     int kv_heads, int dim, int vdim, hipStream_t stream) {
     if (int rc = rec_check("gated_delta_rule", out, state, entry_q_start, entry_seat, entries, heads, kv_heads, dim, vdim)) return rc;
-    KVA_REQUIRE(qkv && y && a_log && dt_bias, "gated_delta_rule: missing operand");
+    // the decay: one per head, formed here from a column of y, a rate and a bias - or one per head and
+    // key channel, handed in ready-made (fp32 [T, >= heads * dim])
+    KVA_REQUIRE(qkv && y && ((a_log && dt_bias) || (channel_decay && decay_stride >= heads * dim)),
+                "gated_delta_rule: missing operand");
     if (entries == 0) return KVA_OK;
     if (dim <= 128) {
         RecArgs a{out, state, (size_t)seat_stride, state_off, entry_q_start, entry_seat, heads, kv_heads, dim, vdim, REC_CHUNK};
         const dim3 grid(heads * ((vdim + REG_BLOCK_COLS - 1) / REG_BLOCK_COLS), entries);
 #define KVA_DELTA_REG(RP)                                                                                              \
-    hipLaunchKernelGGL(gated_delta_rule_reg_kernel<RP>, grid, dim3(REG_THREADS), 0, stream, a, qkv, conv_stride, y,       \
-                       y_dtype, y_stride, beta_off, decay_off, a_log, dt_bias, unit_eps)
+    do {                                                                                                               \
+        if (channel_decay)                                                                                             \
+            hipLaunchKernelGGL((gated_delta_rule_reg_kernel<RP, true>), grid, dim3(REG_THREADS), 0, stream, a, qkv,      \
+                               conv_stride, y, y_dtype, y_stride, beta_off, decay_off, a_log, dt_bias, unit_eps,      \
+                               channel_decay, decay_stride);                                                           \
+        else                                                                                                           \
+            hipLaunchKernelGGL((gated_delta_rule_reg_kernel<RP, false>), grid, dim3(REG_THREADS), 0, stream, a, qkv,     \
+                               conv_stride, y, y_dtype, y_stride, beta_off, decay_off, a_log, dt_bias, unit_eps,      \
+                               channel_decay, decay_stride);                                                           \
+    } while (0)
         if (dim <= 64) KVA_DELTA_REG(4);
         else KVA_DELTA_REG(8);
 #undef KVA_DELTA_REG
         KVA_CHECK_LAUNCH("gated_delta_rule");
         return KVA_OK;
     }
-    const int chunk = rec_chunk(dim, 2);
+    const int arrays = channel_decay ? 3 : 2;
+    const int chunk = rec_chunk(dim, arrays);
     KVA_REQUIRE(chunk > 0, "gated_delta_rule: key size %d does not fit the LDS", dim);
     RecArgs a{out, state, (size_t)seat_stride, state_off, entry_q_start, entry_seat, heads, kv_heads, dim, vdim, chunk};
-    const size_t lds = ((size_t)dim * REC_COLS + (size_t)chunk * dim * 2 + 2 * chunk) * sizeof(float);
+    const size_t lds = ((size_t)dim * REC_COLS + (size_t)chunk * dim * arrays + 2 * chunk) * sizeof(float);
     const int slices = (vdim + REC_COLS - 1) / REC_COLS;
     hipLaunchKernelGGL(gated_delta_rule_kernel, dim3(heads * slices, entries), dim3(KVA_WAVE), lds, stream, a, qkv,
-                       conv_stride, y, y_dtype, y_stride, beta_off, decay_off, a_log, dt_bias, unit_eps);
+                       conv_stride, y, y_dtype, y_stride, beta_off, decay_off, a_log, dt_bias, unit_eps, channel_decay,
+                       decay_stride);
     KVA_CHECK_LAUNCH("gated_delta_rule");
     return KVA_OK;
 }
@@ -612,17 +667,20 @@ extern "C" int kva_gated_delta_rule(float *out, float *state, long long seat_str
 extern "C" int kva_gated_linear_attention(float *out, float *state, long long seat_stride, int state_off,
                                           const void *y, int y_dtype, int y_stride, int q_off, int k_off, int v_off,
                                           const float *alpha, int alpha_stride, float q_mul,
+                                          const float *head_decay, int act,
                                           const int *entry_q_start, const int *entry_seat,
                                           int entries, int heads, int dim, int vdim, hipStream_t stream) {
     if (int rc = rec_check("gated_linear_attention", out, state, entry_q_start, entry_seat, entries, heads, heads, dim, vdim)) return rc;
-    KVA_REQUIRE(y && alpha && alpha_stride >= heads * dim, "gated_linear_attention: missing operand");
+    // the decays: a buffer with one value per token, head and key channel, or one fixed value a head
+    KVA_REQUIRE(y && ((alpha && alpha_stride >= heads * dim) || (!alpha && head_decay)), "gated_linear_attention: missing operand");
+    KVA_REQUIRE(act == 0 || act == 1, "gated_linear_attention: activation %d is neither none (0) nor silu (1)", act);
     if (entries == 0) return KVA_OK;
     if (dim <= 128) {
         RecArgs a{out, state, (size_t)seat_stride, state_off, entry_q_start, entry_seat, heads, heads, dim, vdim, REC_CHUNK};
         const dim3 grid(heads * ((vdim + REG_BLOCK_COLS - 1) / REG_BLOCK_COLS), entries);
 #define KVA_GLA_REG(RP)                                                                                                \
     hipLaunchKernelGGL(gated_linear_attention_reg_kernel<RP>, grid, dim3(REG_THREADS), 0, stream, a, y, y_dtype,          \
-                       y_stride, q_off, k_off, v_off, alpha, alpha_stride, q_mul)
+                       y_stride, q_off, k_off, v_off, alpha, alpha_stride, q_mul, head_decay, act)
         if (dim <= 64) KVA_GLA_REG(4);
         else KVA_GLA_REG(8);
 #undef KVA_GLA_REG
@@ -635,7 +693,7 @@ extern "C" int kva_gated_linear_attention(float *out, float *state, long long se
     const size_t lds = ((size_t)dim * REC_COLS + (size_t)chunk * dim * 3) * sizeof(float);
     const int slices = (vdim + REC_COLS - 1) / REC_COLS;
     hipLaunchKernelGGL(gated_linear_attention_kernel, dim3(heads * slices, entries), dim3(KVA_WAVE), lds, stream, a, y,
-                       y_dtype, y_stride, q_off, k_off, v_off, alpha, alpha_stride, q_mul);
+                       y_dtype, y_stride, q_off, k_off, v_off, alpha, alpha_stride, q_mul, head_decay, act);
     KVA_CHECK_LAUNCH("gated_linear_attention");
     return KVA_OK;
 }

@@ -175,3 +175,74 @@ extern "C" int kva_head_gate(void *x, const void *g, int rows, int heads, int he
     KVA_CHECK_LAUNCH("head_gate");
     return KVA_OK;
 }
+
+// ---- a branch output that is normed before it enters the stream --------------------------------
+// x[t] += y[t] / sqrt(mean(y[t]^2) + eps) * w (an RMS norm on the branch's OUTPUT; the stream itself
+// is read by the branches as it is).  With `copy` the new row of the stream is also written in a
+// second type: what the next branch's products read.  One workgroup a row; the sum of squares is
+// taken in a fixed order.
+__global__ void __launch_bounds__(256)
+norm_into_stream_kernel(void *__restrict__ x, int x_dtype, const void *__restrict__ y, int y_dtype,
+                        const void *__restrict__ w, int w_dtype, void *__restrict__ copy, int copy_dtype, int width,
+                        float eps) {
+    extern __shared__ float row_s[];
+    __shared__ float red_s[4];
+    const size_t at = (size_t)blockIdx.x * width;
+    float sq = 0.f;
+    for (int j = threadIdx.x; j < width; j += blockDim.x) {
+        const float v = ld_as_float(y, y_dtype, at + j);
+        row_s[j] = v;
+        sq += v * v;
+    }
+    const float inv = 1.0f / sqrtf(block_sum(sq, red_s, blockDim.x / KVA_WAVE) / (float)width + eps);
+    for (int j = threadIdx.x; j < width; j += blockDim.x) {
+        const float v = ld_as_float(x, x_dtype, at + j) + row_s[j] * inv * ld_as_float(w, w_dtype, j);
+        st_from_float(x, x_dtype, at + j, v);
+        if (copy) st_from_float(copy, copy_dtype, at + j, x_dtype == KVA_F32 ? v : ld_as_float(x, x_dtype, at + j));
+    }
+}
+
+extern "C" int kva_norm_into_stream(void *x, int x_dtype, const void *y, int y_dtype, const void *w, int w_dtype,
+                                    void *copy, int copy_dtype, int rows, int width, float eps, hipStream_t stream) {
+    KVA_REQUIRE(rows >= 0 && width > 0 && width <= 16000, "norm_into_stream: width %d must lie in 1..16000", width);
+    KVA_REQUIRE(x && y && w && eps >= 0.f, "norm_into_stream: missing operand or negative eps");
+    if (rows == 0) return KVA_OK;
+    hipLaunchKernelGGL(norm_into_stream_kernel, dim3(rows), dim3(256), (size_t)width * sizeof(float), stream, x, x_dtype,
+                       y, y_dtype, w, w_dtype, copy, copy_dtype, width, eps);
+    KVA_CHECK_LAUNCH("norm_into_stream");
+    return KVA_OK;
+}
+
+// ---- a gate times a row of a table that the token picks ------------------------------------------
+// out[t, j] = act(z[t, j]) * table[id_t, col0 + j] for j < dim: what a token brings of its own (a
+// slice of a second embedding table) under a gate computed from the stream.  A negative id -1 - r
+// stands for feedback[r], as in the embedding gather.
+__global__ void __launch_bounds__(256)
+table_gate_kernel(void *__restrict__ out, const void *__restrict__ z, int dtype, const void *__restrict__ table,
+                  int table_dtype, int table_width, int table_rows, int col0, const int *__restrict__ ids,
+                  const int *__restrict__ feedback, int dim, int act, int rows) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)rows * dim) return;
+    const size_t t = i / dim;
+    const int j = (int)(i % dim);
+    int id = ids[t];
+    if (id < 0) id = feedback[-1 - id];
+    id = id < 0 ? 0 : (id >= table_rows ? table_rows - 1 : id);
+    const float e = ld_as_float(table, table_dtype, (size_t)id * table_width + col0 + j);
+    st_from_float(out, dtype, i, kva_activate(ld_as_float(z, dtype, i), act) * e);
+}
+
+extern "C" int kva_table_gate(void *out, const void *z, int dtype, const void *table, int table_dtype, int table_width,
+                              int table_rows, int col0, const int *ids, const int *feedback, int rows, int dim, int act,
+                              hipStream_t stream) {
+    KVA_REQUIRE(out && z && table && ids && rows >= 0 && dim > 0 && table_rows > 0, "table_gate: missing operand or bad sizes");
+    KVA_REQUIRE(col0 >= 0 && col0 + dim <= table_width, "table_gate: columns %d..%d lie outside a table row of %d", col0,
+                col0 + dim, table_width);
+    KVA_REQUIRE(act >= KVA_ACT_SILU && act <= KVA_ACT_GELU_TANH, "table_gate: unknown activation %d", act);
+    if (rows == 0) return KVA_OK;
+    const size_t n = (size_t)rows * dim;
+    hipLaunchKernelGGL(table_gate_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, out, z, dtype, table,
+                       table_dtype, table_width, table_rows, col0, ids, feedback, dim, act, rows);
+    KVA_CHECK_LAUNCH("table_gate");
+    return KVA_OK;
+}

@@ -10,10 +10,11 @@ from .. import parts as _parts  # noqa: F401  (registers the built-in part kinds
 from . import llama as _llama   # noqa: F401  (registers LlamaForCausalLM)
 from . import gadopel as _gadopel   # noqa: F401  (registers Gadopel)
 from . import radilix as _radilix   # noqa: F401  (registers Radilix)
+from . import lomodra as _lomodra   # noqa: F401  (registers Lomodra)
 from ..config.registry import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, STREAM_OPS, architecture_for)
 from ..models.spec import LayerCall, ModelSpec, TensorSpec
 from ..ops import kernels as K
-from ..parts.base import Block, KVCacheSpec, KVView, MixerContext, NormedRows, StateSpec
+from ..parts.base import Block, KVCacheSpec, KVView, MixerContext, NormedRows, StateSpec, StreamCopy
 from ..parts.linear import Linear
 
 
@@ -259,6 +260,8 @@ class Model:
         for i, (call, slot) in enumerate(self.calls):
             block = self.blocks[call.layer]
             if call.before is not None:
+                if isinstance(delta, StreamCopy):
+                    delta = None                    # the stream holds everything already
                 if isinstance(delta, NormedRows):
                     raise TypeError("an operation between layers takes the stream, not rows prepared for a norm")
                 if getattr(delta, "scale", 1.0) != 1.0:
@@ -285,6 +288,8 @@ class Model:
         logits = torch.empty((R, self.spec.vocab_size), dtype=torch.float32, device=self.device)
         if R == 0:
             return logits
+        if isinstance(delta, StreamCopy):
+            delta = None
         if isinstance(delta, NormedRows):
             if R == T and batch.logits_for_all_rows:
                 x = delta                    # the head's product finishes the final norm

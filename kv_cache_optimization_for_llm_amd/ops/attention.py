@@ -350,7 +350,7 @@ def rotates_in_kernel(batch, kv, num_q_heads: int, num_kv_heads: int, head_dim: 
 
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads: int,
                     num_kv_heads: int, head_dim: int, scale: float, window: int = 0, rope=None,
-                    max_parts: int = 0, keep_first: int = 0, sinks=None, value_dim: int = None):
+                    max_parts: int = 0, keep_first: int = 0, sinks=None, value_dim: int = None, chunk: int = 0):
     """Causal GQA attention of the step's tokens over the paged cache.  ``qkv`` is the fused
     projection output ``[T, (nq + 2 nkv) d]`` (or just its Q part) whose first ``nq * d`` columns
     are the (already position-encoded) queries; keys and values are read from ``kv``.
@@ -368,19 +368,23 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
     which is then not written) - where the keys are cut that way no merge kernel runs.
 
     ``keep_first`` (with a window: the first so many positions stay visible behind it), ``sinks``
-    (fp32 per query head: one more term exp(sink) in every denominator) and a ``value_dim`` other
-    than ``head_dim`` are taken by a matrix-core kernel of their own (16 rows of (token, head)
+    (fp32 per query head: one more term exp(sink) in every denominator), a ``value_dim`` other
+    than ``head_dim`` and ``chunk`` (positions see each other only inside runs of so many positions
+    counted from 0; not together with a window) are taken by a matrix-core kernel of their own (16 rows of (token, head)
     pairs a wavefront; bf16, head sizes with an instance) or else by the plain kernel."""
     if kv is None:
         raise K.KernelError("paged_attention: the mixer has no cache view")
     value_dim = head_dim if value_dim is None else int(value_dim)
     if window <= 0:
         keep_first = 0
+    chunk = max(0, int(chunk))
+    if chunk > 0 and window > 0:
+        raise K.KernelError("paged_attention: either a window or chunks")
     # the queries may be the first columns of a wider buffer: rows lie ``stride`` elements apart
     stride = qkv.stride(0)
-    if keep_first > 0 or sinks is not None or value_dim != head_dim:
+    if keep_first > 0 or sinks is not None or value_dim != head_dim or chunk > 0:
         if rope is not None or max_parts:
-            raise K.KernelError("paged_attention: kept first positions, sinks and a value size of its own "
+            raise K.KernelError("paged_attention: kept first positions, sinks, chunks and a value size of its own "
                                 "go with neither rotation inside the kernel nor partial results")
         if qkv.dtype == torch.bfloat16 and stride % 8 == 0 \
                 and K.attention_rows_mfma_supported(head_dim, value_dim, kv.page_size):
@@ -392,14 +396,14 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
             item_entry, item_row0, _ = batch.attention_items(group, tiles, "all")
             # (with a window most ranges of a long context hold no visible key: their wavefronts end at once)
             ranges, per = choose_ranges(item_entry.shape[0] * num_kv_heads, batch.max_context,
-                                        window + keep_first if window > 0 else 0)
+                                        window + keep_first if window > 0 else chunk)
             return K.attention_rows_mfma(qkv, stride, out, kv.k_cache, kv.v_cache, kv.block_table, item_entry,
                                          item_row0, batch.entry_seat, batch.entry_q_start, batch.entry_start_pos,
                                          num_q_heads, num_kv_heads, head_dim, scale, window, keep_first, sinks,
-                                         value_dim, ranges, per, tiles)
+                                         value_dim, ranges, per, tiles, chunk)
         return K.attention_rowwise(qkv, stride, out, kv.k_cache, kv.v_cache, kv.block_table,
                                    batch.tok_seat, batch.positions, num_q_heads, num_kv_heads,
-                                   head_dim, scale, window, keep_first, sinks, value_dim)
+                                   head_dim, scale, window, keep_first, sinks, value_dim, chunk)
     if rope is not None:
         # decoded tokens whose rotation and cache write are still to be done: ``rope`` = (cos, sin)
         # tables or (None, None); only where rotates_in_kernel() said yes

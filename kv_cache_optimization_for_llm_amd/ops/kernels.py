@@ -364,10 +364,11 @@ def attention_rowwise(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_c
                       v_cache: torch.Tensor, block_table: torch.Tensor, tok_seat: torch.Tensor,
                       tok_pos: torch.Tensor, num_q_heads: int, num_kv_heads: int, head_dim: int,
                       scale: float, window: int = 0, keep_first: int = 0, sinks: Optional[torch.Tensor] = None,
-                      value_dim: Optional[int] = None) -> torch.Tensor:
+                      value_dim: Optional[int] = None, chunk: int = 0) -> torch.Tensor:
     """Causal GQA attention of every token over its request's cached keys; ``q`` is a view whose
     rows are ``q_row_stride`` elements apart (the Q part of a fused QKV buffer).  With a
-    ``window`` a query at position i sees key j when ``i - j < window`` or ``j < keep_first``;
+    ``window`` a query at position i sees key j when ``i - j < window`` or ``j < keep_first``; with a
+    ``chunk`` when both lie in the same run of ``chunk`` positions counted from 0;
     ``sinks`` (fp32, one per query head) adds ``exp(sink)`` to every softmax denominator;
     ``value_dim`` is the size of a value where it differs from a key's."""
     tokens = out.shape[0]
@@ -389,7 +390,7 @@ def attention_rowwise(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_c
         _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32), block_table.shape[1],
         _dev(tok_seat, "tok_seat", torch.int32), _dev(tok_pos, "tok_pos", torch.int32), tokens,
         num_q_heads, num_kv_heads, head_dim, value_dim, page_size, float(scale), int(window), int(keep_first),
-        _opt(sinks, "sinks"), dtype_code(out.dtype), _stream()), "attention_rowwise")
+        int(chunk), _opt(sinks, "sinks"), dtype_code(out.dtype), _stream()), "attention_rowwise")
     return out
 
 
@@ -477,7 +478,7 @@ def attention_rows_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k
                         entry_start_pos: torch.Tensor, num_q_heads: int, num_kv_heads: int, head_dim: int,
                         scale: float, window: int = 0, keep_first: int = 0, sinks: Optional[torch.Tensor] = None,
                         value_dim: Optional[int] = None, splits: int = 1, per_split: int = 0,
-                        row_tiles: int = 1) -> torch.Tensor:
+                        row_tiles: int = 1, chunk: int = 0) -> torch.Tensor:
     """:func:`attention_rowwise` with all its options on the matrix cores (bf16): a work item is
     ``16 * row_tiles`` rows ``token_in_entry * group + head_in_group`` of entry ``item_entry[i]`` from
     ``item_row0[i]`` on, for every kv head (two row tiles, for heads up to 128, share what a
@@ -511,8 +512,8 @@ def attention_rows_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k
         block_table.shape[1], _dev(item_entry, "item_entry", torch.int32), _dev(item_row0, "item_row0", torch.int32),
         _dev(entry_seat, "entry_seat", torch.int32), _dev(entry_q_start, "entry_q_start", torch.int32),
         _dev(entry_start_pos, "entry_start_pos", torch.int32), n, tokens * num_q_heads, num_q_heads, num_kv_heads,
-        head_dim, value_dim, page_size, float(scale), int(window), int(keep_first), _opt(sinks, "sinks"), int(splits),
-        int(per_split), int(row_tiles), _stream()), "attention_rows_mfma")
+        head_dim, value_dim, page_size, float(scale), int(window), int(keep_first), int(chunk), _opt(sinks, "sinks"),
+        int(splits), int(per_split), int(row_tiles), _stream()), "attention_rows_mfma")
     return out
 
 
@@ -567,7 +568,39 @@ def stream_join(x: torch.Tensor, other: torch.Tensor, out: torch.Tensor, deltas=
     return out
 
 
+def norm_into_stream(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float,
+                     copy: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """In place: ``x += y / sqrt(mean(y^2) + eps) * weight`` per row - a branch's output normed on its
+    way into the stream.  ``x`` (the stream) and ``y`` may be of different storage types; ``copy``
+    (x's shape, any storage type) receives the new rows of the stream as well."""
+    if x.dim() != 2 or y.shape != x.shape or weight.shape != (x.shape[1],) or (copy is not None and copy.shape != x.shape):
+        raise KernelError(f"norm_into_stream: x {tuple(x.shape)}, y {tuple(y.shape)}, weight {tuple(weight.shape)} do not fit")
+    check(hip_lib().kva_norm_into_stream(
+        _dev(x, "x"), dtype_code(x.dtype), _dev(y, "y"), dtype_code(y.dtype), _dev(weight, "weight"), dtype_code(weight.dtype),
+        _opt(copy, "copy"), dtype_code(copy.dtype) if copy is not None else 0, x.shape[0], x.shape[1], float(eps),
+        _stream()), "norm_into_stream")
+    return x
+
+
 ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2}
+
+
+def table_gate(z: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, col0: int, out: torch.Tensor, activation: str,
+               feedback: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out[t, j] = act(z[t, j]) * table[ids[t], col0 + j]``: a gate times the columns ``col0 ..`` of the
+    table row the token picks.  A negative id ``-1 - r`` stands for ``feedback[r]`` as in
+    :func:`embed_gather`."""
+    rows, dim = z.shape
+    if activation not in ACTIVATIONS:
+        raise KernelError(f"table_gate: activation {activation!r} is not one of {sorted(ACTIVATIONS)}")
+    if out.shape != z.shape or out.dtype != z.dtype or table.dim() != 2 or ids.shape != (rows,) \
+            or not 0 <= col0 <= table.shape[1] - dim:
+        raise KernelError(f"table_gate: z {tuple(z.shape)}, table {tuple(table.shape)}, columns from {col0} do not fit")
+    check(hip_lib().kva_table_gate(
+        _dev(out, "out"), _dev(z, "z"), dtype_code(z.dtype), _dev(table, "table"), dtype_code(table.dtype), table.shape[1],
+        table.shape[0], int(col0), _dev(ids, "ids", torch.int32), _opt(feedback, "feedback", torch.int32), rows, dim,
+        ACTIVATIONS[activation], _stream()), "table_gate")
+    return out
 
 
 def act_mul(gate_up: torch.Tensor, out: torch.Tensor, activation: str) -> torch.Tensor:
@@ -599,14 +632,24 @@ def head_gate(x: torch.Tensor, gates: torch.Tensor, heads: int) -> torch.Tensor:
 def qk_encode_cache(qkv: torch.Tensor, positions: torch.Tensor, num_q_heads: int, num_kv_heads: int, head_dim: int,
                     value_dim: int, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], interleaved: bool,
                     unit_eps: Optional[float], k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
-                    slot_mapping: Optional[torch.Tensor], bias: Optional[torch.Tensor] = None) -> None:
+                    slot_mapping: Optional[torch.Tensor], bias: Optional[torch.Tensor] = None,
+                    q_weight: Optional[torch.Tensor] = None, k_weight: Optional[torch.Tensor] = None) -> None:
     """Rotates the first ``2 * cos.shape[1]`` elements of every Q and K head of ``qkv``
     ``[T, nq d + nkv d + nkv value_dim]`` (pair i = elements (2i, 2i + 1) when ``interleaved``, else
     (i, i + rot / 2)), then - with ``unit_eps`` - divides every head by its root mean square; Q in
     place, K and the plain V into the paged cache at ``slot_mapping``.  ``qkv`` may be the first
     columns of a wider buffer (rows ``qkv.stride(0)`` apart).  ``bias`` (qkv's type, one value per
-    column) is added to Q, K and V first: the projection's bias, applied here."""
+    column) is added to Q, K and V first: the projection's bias, applied here.  ``q_weight`` /
+    ``k_weight`` (fp32 ``[head_dim]``, with ``unit_eps``): every query / key head is multiplied by it
+    after the division - an RMS norm of the head with a weight shared by the heads.
+    ``num_kv_heads = 0``: ``qkv`` holds queries alone (a layer that reads another layer's keys and
+    values); nothing is written to a cache."""
     tokens = qkv.shape[0]
+    for w in (q_weight, k_weight):
+        if w is not None and (unit_eps is None or w.shape != (head_dim,) or w.dtype != torch.float32):
+            raise KernelError("qk_encode_cache: a head's norm weight is fp32 [head_dim] and goes with unit_eps")
+    if num_kv_heads == 0 and k_cache is not None:
+        raise KernelError("qk_encode_cache: rows of queries alone write no cache")
     k_off = num_q_heads * head_dim
     v_off = k_off + num_kv_heads * head_dim
     if qkv.dim() != 2 or qkv.shape[1] != v_off + num_kv_heads * value_dim or positions.shape != (tokens,) \
@@ -632,7 +675,8 @@ def qk_encode_cache(qkv: torch.Tensor, positions: torch.Tensor, num_q_heads: int
         _opt(cos, "cos", torch.float32), _opt(sin, "sin", torch.float32), _dev(positions, "positions", torch.int32),
         _opt(slot_mapping if write else None, "slot_mapping", torch.int32), tokens, num_q_heads, num_kv_heads,
         head_dim, value_dim, rot, 1 if interleaved else 0, -1.0 if unit_eps is None else float(unit_eps),
-        page_size, dtype_code(qkv.dtype), _opt(bias, "bias"), _stream()), "qk_encode_cache")
+        page_size, dtype_code(qkv.dtype), _opt(bias, "bias"), _opt(q_weight, "q_weight"), _opt(k_weight, "k_weight"),
+        _stream()), "qk_encode_cache")
 
 
 def latent_encode_cache(y: torch.Tensor, kv_off: int, q_lat: torch.Tensor, cache: Optional[torch.Tensor],
@@ -1399,45 +1443,66 @@ def causal_conv_act(y: torch.Tensor, col_off: int, weight: torch.Tensor, out: to
     return out
 
 
-def gated_delta_rule(qkv: torch.Tensor, y: torch.Tensor, beta_off: int, decay_off: int, a_log: torch.Tensor,
-                     dt_bias: torch.Tensor, out: torch.Tensor, state: torch.Tensor, state_off: int,
+def gated_delta_rule(qkv: torch.Tensor, y: torch.Tensor, beta_off: int, decay_off: int, a_log: Optional[torch.Tensor],
+                     dt_bias: Optional[torch.Tensor], out: torch.Tensor, state: torch.Tensor, state_off: int,
                      entry_q_start: torch.Tensor, entry_seat: torch.Tensor, heads: int, kv_heads: int, dim: int,
-                     vdim: int, unit_eps: float = 1e-6) -> torch.Tensor:
+                     vdim: int, unit_eps: float = 1e-6, channel_decay: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Per head and token, in order: ``S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q`` with
     q and k made unit vectors (``x / sqrt(sum x^2 + unit_eps)``, q also times ``dim^-1/2``),
     ``beta = sigmoid(y[t, beta_off + h])`` and ``g = exp(-exp(a_log[h]) softplus(y[t, decay_off + h] +
     dt_bias[h]))``.  ``qkv`` fp32 ``[T, 2 kv_heads dim + heads vdim]`` holds q, k (``kv_heads`` heads) and v;
     head h uses q/k head ``h // (heads / kv_heads)``.  ``S`` ``[heads, dim, vdim]`` lives at ``state_off`` of
-    the seat's fp32 state row.  ``out`` fp32 ``[T, heads * vdim]``."""
+    the seat's fp32 state row.  ``out`` fp32 ``[T, heads * vdim]``.
+
+    ``channel_decay`` (fp32 ``[T, heads * dim]``, e.g. from :func:`small_product_f32` with ``rate_log``):
+    the decay has one value per head and key channel and multiplies the rows of ``S`` one by one,
+    ``S <- diag(g) S``; ``decay_off``, ``a_log`` and ``dt_bias`` are then not used."""
     tokens = out.shape[0]
     if qkv.shape != (tokens, 2 * kv_heads * dim + heads * vdim) or qkv.dtype != torch.float32 \
             or out.shape != (tokens, heads * vdim) or out.dtype != torch.float32 or y.dim() != 2 or y.shape[0] != tokens:
         raise KernelError(f"gated_delta_rule: qkv {tuple(qkv.shape)}, y {tuple(y.shape)}, out {tuple(out.shape)} do not fit")
-    if not (0 <= beta_off <= y.shape[1] - heads and 0 <= decay_off <= y.shape[1] - heads):
-        raise KernelError("gated_delta_rule: beta and decay columns lie outside y")
-    if a_log.shape != (heads,) or dt_bias.shape != (heads,):
-        raise KernelError("gated_delta_rule: one rate and one bias per head")
+    if not 0 <= beta_off <= y.shape[1] - heads:
+        raise KernelError("gated_delta_rule: beta columns lie outside y")
+    if channel_decay is not None:
+        if channel_decay.shape != (tokens, heads * dim) or channel_decay.dtype != torch.float32:
+            raise KernelError(f"gated_delta_rule: decays per channel are fp32 [T, heads * dim], got {tuple(channel_decay.shape)}")
+        decay_off = 0
+    elif not 0 <= decay_off <= y.shape[1] - heads or a_log is None or dt_bias is None \
+            or a_log.shape != (heads,) or dt_bias.shape != (heads,):
+        raise KernelError("gated_delta_rule: decay columns inside y, one rate and one bias per head")
     seat_stride = _state_row(state, state_off, heads * dim * vdim, "gated_delta_rule")
     qs, seat, entries = _entries((entry_q_start, entry_seat), "gated_delta_rule")
     check(hip_lib().kva_gated_delta_rule(
         _dev(out, "out"), _dev(state, "state"), seat_stride, int(state_off), _dev(qkv, "qkv"), qkv.shape[1],
         _dev(y, "y"), dtype_code(y.dtype), y.shape[1], int(beta_off), int(decay_off),
-        _dev(a_log, "a_log", torch.float32), _dev(dt_bias, "dt_bias", torch.float32), float(unit_eps), qs, seat,
+        _opt(a_log, "a_log", torch.float32), _opt(dt_bias, "dt_bias", torch.float32), float(unit_eps),
+        _opt(channel_decay, "channel_decay"), channel_decay.shape[1] if channel_decay is not None else 0, qs, seat,
         entries, heads, kv_heads, dim, vdim, _stream()), "gated_delta_rule")
     return out
 
 
-def gated_linear_attention(y: torch.Tensor, q_off: int, k_off: int, v_off: int, alpha: torch.Tensor, q_mul: float,
+def gated_linear_attention(y: torch.Tensor, q_off: int, k_off: int, v_off: int, alpha: Optional[torch.Tensor], q_mul: float,
                            out: torch.Tensor, state: torch.Tensor, state_off: int, entry_q_start: torch.Tensor,
-                           entry_seat: torch.Tensor, heads: int, dim: int, vdim: int) -> torch.Tensor:
+                           entry_seat: torch.Tensor, heads: int, dim: int, vdim: int,
+                           head_decay: Optional[torch.Tensor] = None, activation: Optional[str] = None) -> torch.Tensor:
     """Per head and token, in order: ``S <- diag(alpha) S + k v^T; o = S^T (q_mul q)`` with a decay per
     key channel ``alpha`` (fp32 ``[T, heads * dim]``; :func:`small_product_f32` makes it from a low-rank
     projection).  q, k (``heads x dim``) and v (``heads x vdim``) are columns of ``y`` from ``q_off``,
-    ``k_off``, ``v_off`` on.  ``out`` fp32 ``[T, heads * vdim]``."""
+    ``k_off``, ``v_off`` on.  ``out`` fp32 ``[T, heads * vdim]``.
+
+    ``alpha=None`` with ``head_decay`` (fp32 ``[heads]``): one fixed decay a head for all its channels
+    and every token, ``S <- decay_h S + k v^T``.  ``activation="silu"``: q, k and v pass a silu (in
+    fp32) on their way in."""
     tokens = out.shape[0]
-    if y.dim() != 2 or y.shape[0] != tokens or out.shape != (tokens, heads * vdim) or out.dtype != torch.float32 \
-            or alpha.shape != (tokens, heads * dim) or alpha.dtype != torch.float32:
-        raise KernelError(f"gated_linear_attention: y {tuple(y.shape)}, alpha {tuple(alpha.shape)}, out {tuple(out.shape)} do not fit")
+    if y.dim() != 2 or y.shape[0] != tokens or out.shape != (tokens, heads * vdim) or out.dtype != torch.float32:
+        raise KernelError(f"gated_linear_attention: y {tuple(y.shape)}, out {tuple(out.shape)} do not fit")
+    if alpha is not None:
+        if alpha.shape != (tokens, heads * dim) or alpha.dtype != torch.float32 or head_decay is not None:
+            raise KernelError(f"gated_linear_attention: alpha {tuple(alpha.shape)} is fp32 [T, heads * dim], without fixed decays")
+    elif head_decay is None or head_decay.shape != (heads,) or head_decay.dtype != torch.float32:
+        raise KernelError("gated_linear_attention: decays per token and channel, or one fp32 value a head")
+    if activation not in (None, "silu"):
+        raise KernelError(f"gated_linear_attention: activation {activation!r} is neither None nor 'silu'")
     for off, n in ((q_off, heads * dim), (k_off, heads * dim), (v_off, heads * vdim)):
         if not 0 <= off <= y.shape[1] - n:
             raise KernelError("gated_linear_attention: q, k or v columns lie outside y")
@@ -1445,7 +1510,8 @@ def gated_linear_attention(y: torch.Tensor, q_off: int, k_off: int, v_off: int, 
     qs, seat, entries = _entries((entry_q_start, entry_seat), "gated_linear_attention")
     check(hip_lib().kva_gated_linear_attention(
         _dev(out, "out"), _dev(state, "state"), seat_stride, int(state_off), _dev(y, "y"), dtype_code(y.dtype),
-        y.shape[1], int(q_off), int(k_off), int(v_off), _dev(alpha, "alpha"), alpha.shape[1], float(q_mul), qs, seat,
+        y.shape[1], int(q_off), int(k_off), int(v_off), _opt(alpha, "alpha"), alpha.shape[1] if alpha is not None else 0,
+        float(q_mul), _opt(head_decay, "head_decay"), 1 if activation == "silu" else 0, qs, seat,
         entries, heads, dim, vdim, _stream()), "gated_linear_attention")
     return out
 
@@ -1482,17 +1548,18 @@ EXPERT_ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2, "gelu": 3}
 
 
 def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, idx: torch.Tensor,
-              wgt: torch.Tensor, renormalise: bool = False) -> None:
+              wgt: torch.Tensor, renormalise: bool = False, over_chosen: bool = False) -> None:
     """``scores = softmax(logits)`` over all router outputs; the ``top`` largest of ``scores +
     correction`` are chosen (of equal ones the lowest index) into ``idx`` ``[T, top]``; ``wgt`` gets their
-    plain scores, divided by their sum with ``renormalise``."""
+    plain scores, divided by their sum with ``renormalise``.  ``over_chosen``: the ``top`` largest
+    logits (plus correction) are chosen and the weights are the softmax over the chosen logits alone."""
     tokens, outputs = logits.shape
     if logits.dtype != torch.float32 or idx.shape != (tokens, top) or wgt.shape != (tokens, top) \
             or (correction is not None and correction.shape != (outputs,)):
         raise KernelError(f"moe_route: logits {tuple(logits.shape)}, idx {tuple(idx.shape)}, wgt {tuple(wgt.shape)} do not fit")
     check(hip_lib().kva_moe_route(_dev(idx, "idx", torch.int32), _dev(wgt, "wgt", torch.float32), _dev(logits, "logits"),
                                   _opt(correction, "correction", torch.float32), tokens, outputs, int(top),
-                                  1 if renormalise else 0, _stream()), "moe_route")
+                                  1 if renormalise else 0, 1 if over_chosen else 0, _stream()), "moe_route")
 
 
 def moe_tiles(slots: int, experts: int) -> int:
@@ -1514,17 +1581,21 @@ def moe_align(idx: torch.Tensor, experts: int, sorted_slot: torch.Tensor, tile_e
 
 def moe_expert_rows(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, sorted_slot: torch.Tensor,
                     tile_expert: torch.Tensor, top: int, *, activation: Optional[str] = None,
-                    slot_weight: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    slot_weight: Optional[torch.Tensor] = None, gated: bool = False) -> torch.Tensor:
     """One product per tile against its expert's matrix ``w[e]`` ``[N, K]``.  With an ``activation``
     (the first product): row ``slot // top`` of ``x`` ``[T, K]``, activated, goes to the slot's sorted
     place of ``out`` ``[places, N]`` (x's type).  With ``slot_weight`` (the second): the row at the
     sorted place of ``x`` ``[places, K]``, times the slot's weight, goes to row ``slot`` of ``out`` fp32
-    ``[slots, N]``."""
+    ``[slots, N]``.  ``gated`` (first product): rows ``2 j`` and ``2 j + 1`` of an expert's matrix are
+    output j's gate and up rows, and ``out`` ``[places, N / 2]`` gets ``act(gate) * up``."""
     tiles = tile_expert.shape[0]
+    n_out = w.shape[1] // 2 if gated else w.shape[1]
+    if gated and (activation is None or w.shape[1] % 2):
+        raise KernelError("moe_expert_rows: gate and up rows come in pairs, in the first product")
     if (activation is None) == (slot_weight is None):
         raise KernelError("moe_expert_rows: either an activation (first product) or slot weights (second)")
     if w.dim() != 3 or w.dtype != x.dtype or x.dim() != 2 or x.shape[1] != w.shape[2] or out.dim() != 2 \
-            or out.shape[1] != w.shape[1] or sorted_slot.shape != (tiles * MOE_TILE,):
+            or out.shape[1] != n_out or sorted_slot.shape != (tiles * MOE_TILE,):
         raise KernelError(f"moe_expert_rows: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
     if activation is not None:
         if activation not in EXPERT_ACTIVATIONS:
@@ -1539,7 +1610,7 @@ def moe_expert_rows(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, sorted_
         _dev(out, "out"), dtype_code(out.dtype), _dev(x, "x"), _dev(w, "w"), dtype_code(x.dtype),
         _dev(sorted_slot, "sorted_slot", torch.int32), _dev(tile_expert, "tile_expert", torch.int32),
         _opt(slot_weight, "slot_weight"), tiles, int(top), w.shape[1], w.shape[2], 0 if activation is not None else 1,
-        EXPERT_ACTIVATIONS.get(activation, 0), _stream()), "moe_expert_rows")
+        EXPERT_ACTIVATIONS.get(activation, 0), 1 if gated else 0, _stream()), "moe_expert_rows")
     return out
 
 
@@ -1547,12 +1618,17 @@ SMALL_PRODUCT_MAX_K = 8192
 
 
 def small_product_f32(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
-                      decay_tau: float = 0.0) -> torch.Tensor:
+                      decay_tau: float = 0.0, rate_log: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``out = x @ w^T (+ bias)`` with fp32 products, sums and results, for small matrices whose results must
     not be rounded to 16 bits (a router's logits, the second half of a low-rank projection that makes
     decays).  With ``decay_tau`` > 0 the result is turned into a decay, ``sigmoid(.)^(1 / decay_tau)``.
+    With ``rate_log`` (fp32 ``[G]``, G dividing N) it is turned into ``exp(-exp(rate_log[n // (N / G)]) *
+    softplus(.))``: a decay per output whose rate is shared by runs of neighbouring outputs.
     ``x`` ``[T, K]`` may be columns of a wider buffer; ``x`` and ``w`` ``[N, K]`` are bf16 or fp32."""
     tokens, k = x.shape
+    if rate_log is not None and (rate_log.dim() != 1 or rate_log.dtype != torch.float32 or w.shape[0] % rate_log.shape[0]
+                                 or decay_tau > 0):
+        raise KernelError("small_product_f32: rates are fp32, one per run of outputs, and exclude decay_tau")
     if bias is not None and (bias.shape != (w.shape[0],) or bias.dtype != torch.float32):
         raise KernelError("small_product_f32: the bias is fp32, one value per output")
     if w.dim() != 2 or w.shape[1] != k or out.shape != (tokens, w.shape[0]) or out.dtype != torch.float32 \
@@ -1561,22 +1637,25 @@ def small_product_f32(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias:
     check(hip_lib().kva_small_product_f32(
         _dev(out, "out"), _dev(x, "x", contiguous=False), dtype_code(x.dtype), x.stride(0) if tokens > 1 else k,
         _dev(w, "w"), dtype_code(w.dtype), tokens, w.shape[0], k, _opt(bias, "bias"),
-        1.0 / float(decay_tau) if decay_tau > 0 else 0.0, _stream()), "small_product_f32")
+        1.0 / float(decay_tau) if decay_tau > 0 else 0.0, _opt(rate_log, "rate_log"),
+        w.shape[0] // rate_log.shape[0] if rate_log is not None else 0, _stream()), "small_product_f32")
     return out
 
 
 def moe_combine(x: torch.Tensor, rows: torch.Tensor, idx: torch.Tensor, wgt: torch.Tensor, experts: int,
-                out: torch.Tensor) -> torch.Tensor:
+                out: torch.Tensor, extra: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``out[t] = sum over the token's choices`` of the slot's row of ``rows`` (fp32 ``[T * top, width]``,
-    already weighted) or, for a choice past the real ``experts`` (an identity expert), ``wgt * x[t]``."""
+    already weighted) or, for a choice past the real ``experts`` (an identity expert), ``wgt * x[t]``;
+    ``extra`` (x's shape and type: what an expert that every token uses returned) is added last."""
     tokens, width = x.shape
     top = idx.shape[1]
     if out.shape != x.shape or out.dtype != x.dtype or rows.shape != (tokens * top, width) or rows.dtype != torch.float32 \
-            or idx.shape != (tokens, top) or wgt.shape != (tokens, top):
+            or idx.shape != (tokens, top) or wgt.shape != (tokens, top) \
+            or (extra is not None and (extra.shape != x.shape or extra.dtype != x.dtype)):
         raise KernelError(f"moe_combine: x {tuple(x.shape)}, rows {tuple(rows.shape)}, idx {tuple(idx.shape)} do not fit")
     check(hip_lib().kva_moe_combine(_dev(out, "out"), _dev(x, "x"), dtype_code(x.dtype), _dev(rows, "rows"),
-                                    _dev(idx, "idx", torch.int32), _dev(wgt, "wgt", torch.float32), tokens, width, top,
-                                    int(experts), _stream()), "moe_combine")
+                                    _dev(idx, "idx", torch.int32), _dev(wgt, "wgt", torch.float32), _opt(extra, "extra"),
+                                    tokens, width, top, int(experts), _stream()), "moe_combine")
     return out
 
 
@@ -1600,6 +1679,7 @@ KERNEL_CLASSES = {
     "gated_linear_attention": "recurrent mixers", "head_norm_gate": "elementwise",
     "moe_route": "routed experts", "moe_align": "routed experts", "moe_expert_rows": "routed experts",
     "moe_combine": "routed experts", "small_product_f32": "small fp32 products",
+    "norm_into_stream": "norm", "table_gate": "elementwise",
 }
 
 

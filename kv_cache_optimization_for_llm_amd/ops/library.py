@@ -43,17 +43,17 @@ _HIP_SIGNATURES = {
     "kva_silu_mul": [P, P, I, I, I, P],
     "kva_cast": [P, P, LL, I, I, P],
     "kva_rope_kv_write": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
-    "kva_attention_rowwise": [P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P, I, P],
+    "kva_attention_rowwise": [P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, I, P, I, P],
     "kva_latent_attention_rowwise": [P, P, P, P, I, P, P, I, I, I, I, I, F, I, I, P, I, P],
     "kva_layernorm": [P, P, I, P, I, P, I, P, I, P, P, I, P, I, I, F, I, F, P],
     "kva_stream_join": [P, I, P, I, P, I, P, I, P, I, I, I, I, P],
     "kva_act_mul": [P, P, I, I, I, I, P],
     "kva_head_gate": [P, P, I, I, I, I, I, P],
-    "kva_qk_encode_cache": [P, I, I, I, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, P],
+    "kva_qk_encode_cache": [P, I, I, I, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, P, P, P],
     "kva_latent_encode_cache": [P, I, I, P, P, P, I, P, I, F, P, P, P, P, I, I, I, I, I, I, I, P],
     "kva_latent_attention_mfma_supported": [I, I, I],
     "kva_attention_rows_mfma_supported": [I, I, I],
-    "kva_attention_rows_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, I, I, I, P],
+    "kva_attention_rows_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P, I, I, I, P],
     "kva_latent_attention_mfma": [P, P, P, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P, I, I, P],
     "kva_heads_matmul": [P, I, I, P, I, I, P, I, I, I, I, P, I, I, P],
     "kva_heads_matmul_mfma_supported": [I, I, I],
@@ -92,14 +92,16 @@ _HIP_SIGNATURES = {
     "kva_sample": [P, P, I, I, I, P, P, F, P, U, P, P, I, P, P, P, P, P],
     "kva_mark_tokens": [P, P, P, I, I, P],
     "kva_causal_conv_act": [P, I, P, I, I, I, P, I, P, LL, I, P, P, I, I, I, I, P],
-    "kva_gated_delta_rule": [P, P, LL, I, P, I, P, I, I, I, I, P, P, F, P, P, I, I, I, I, I, P],
-    "kva_gated_linear_attention": [P, P, LL, I, P, I, I, I, I, I, P, I, F, P, P, I, I, I, I, P],
+    "kva_gated_delta_rule": [P, P, LL, I, P, I, P, I, I, I, I, P, P, F, P, I, P, P, I, I, I, I, I, P],
+    "kva_gated_linear_attention": [P, P, LL, I, P, I, I, I, I, I, P, I, F, P, I, P, P, I, I, I, I, P],
     "kva_head_norm_gate": [P, I, I, I, P, I, P, F, P, I, I, I, I, I, I, I, F, P],
-    "kva_moe_route": [P, P, P, P, I, I, I, I, P],
+    "kva_moe_route": [P, P, P, P, I, I, I, I, I, P],
     "kva_moe_align": [P, P, P, I, I, I, I, P],
-    "kva_moe_expert_rows": [P, I, P, P, I, P, P, P, I, I, I, I, I, I, P],
-    "kva_moe_combine": [P, P, I, P, P, P, I, I, I, I, P],
-    "kva_small_product_f32": [P, P, I, I, P, I, I, I, I, P, F, P],
+    "kva_moe_expert_rows": [P, I, P, P, I, P, P, P, I, I, I, I, I, I, I, P],
+    "kva_moe_combine": [P, P, I, P, P, P, P, I, I, I, I, P],
+    "kva_small_product_f32": [P, P, I, I, P, I, I, I, I, P, F, P, I, P],
+    "kva_norm_into_stream": [P, I, P, I, P, I, P, I, I, I, F, P],
+    "kva_table_gate": [P, P, I, P, I, I, I, I, P, P, I, I, I, P],
 }
 
 

@@ -268,3 +268,90 @@ class GatedGQAAttention(ProjectedMixer):
             else:
                 K.head_norm_gate(heads, None, 0.0, y, col0 + self.qkv_width, out, out_col0, self.num_heads,
                                  self.value_dim, self.gate, mul)
+
+
+@MIXERS.register("normed_gqa_attention")
+class NormedGQAAttention(Mixer):
+    """Grouped-query causal attention whose queries and keys pass an RMS norm per head (a weight
+    of ``head_dim`` elements for the queries and one for the keys, shared by the heads) before the
+    scores are taken: ``q <- q / sqrt(mean(q^2) + eps) * w_q``, likewise k; the keys lie in the cache
+    normed.  The position encoding is a part as everywhere (``"none"``: positions do not enter the
+    scores); a rotation is applied before the norm.  Masks: all earlier keys, a ``window`` (with kept
+    first positions), or ``chunk``: a query sees a key only inside its own run of ``chunk``
+    positions counted from the request's position 0 - wherever a prompt was cut into steps.
+
+    ``shared_kv``: the mixer has no key and value tensors; it attends, with queries, norm, mask and
+    output matrix of its own, over what another layer call wrote to the cache slot it is given (the
+    run order names that slot with ``writes_cache=False``)."""
+
+    graph_safe = True
+
+    def __init__(self, prefix: str, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 scale: float, norm_eps: float, position: Optional[PartSpec] = None, value_dim: Optional[int] = None,
+                 window: int = 0, keep_first: int = 0, chunk: int = 0, shared_kv: bool = False,
+                 tensor_names: Optional[Dict[str, str]] = None):
+        """``tensor_names`` maps ``q k v o q_norm k_norm`` to names behind ``prefix``."""
+        super().__init__(prefix)
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads is not a multiple of {num_kv_heads} kv heads")
+        if window > 0 and chunk > 0:
+            raise ValueError(f"{prefix}: either a window or chunks")
+        self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.head_dim, self.scale, self.norm_eps = int(head_dim), float(scale), float(norm_eps)
+        self.value_dim = int(head_dim if value_dim is None else value_dim)
+        self.window, self.chunk = int(window), int(chunk)
+        self.keep_first = int(keep_first) if self.window > 0 else 0
+        self.shared_kv = bool(shared_kv)
+        names = dict(q="q", k="k", v="v", o="o", q_norm="q.norm", k_norm="k.norm")
+        names.update(tensor_names or {})
+        self.names = {key: prefix + name for key, name in names.items()}
+        position = position or PartSpec("none")
+        self.position = POSITION_ENCODINGS.get(position.kind)(**position.params)
+        self.in_linear: Optional[Linear] = None
+        self.o: Optional[Linear] = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        n, d, dv, W = self.names, self.head_dim, self.value_dim, self.hidden_size
+        specs = {n["q"]: TensorSpec((self.num_heads * d, W)), n["o"]: TensorSpec((W, self.num_heads * dv)),
+                 n["q_norm"]: TensorSpec((d,), init="norm", role="vector")}
+        if not self.shared_kv:
+            specs[n["k"]] = TensorSpec((self.num_kv_heads * d, W))
+            specs[n["v"]] = TensorSpec((self.num_kv_heads * dv, W))
+            specs[n["k_norm"]] = TensorSpec((d,), init="norm", role="vector")
+        return specs
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        n = self.names
+        rows = [tensors[n["q"]]] if self.shared_kv else [tensors[n[key]] for key in "qkv"]
+        if len({r.dtype for r in rows}) != 1:
+            raise ValueError(f"{self.prefix}: q/k/v projection weights are stored in different dtypes")
+        self.in_linear = Linear(torch.cat(rows, dim=0) if len(rows) > 1 else rows[0])
+        self.o = Linear(tensors[n["o"]])
+        self.q_weight = tensors[n["q_norm"]].float().contiguous()
+        self.k_weight = None if self.shared_kv else tensors[n["k_norm"]].float().contiguous()
+
+    def kv_cache_spec(self) -> KVCacheSpec:
+        # (a chunked layer keeps all its pages: a layer that shares the slot may see them with another mask)
+        return attention_cache_spec(self.num_kv_heads, self.head_dim, kind="window" if self.window > 0 else "full",
+                                    window=self.window, value_dim=self.value_dim, keep_first=self.keep_first)
+
+    def activation_elements(self) -> int:
+        return (self.num_heads + self.num_kv_heads) * (self.head_dim + self.value_dim) + self.hidden_size
+
+    def forward(self, x, ctx: MixerContext):
+        batch, kv = ctx.batch, ctx.kv
+        if kv is None:
+            raise K.KernelError(f"{self.prefix}: the mixer has no cache view")
+        if self.shared_kv and kv.writes:
+            raise K.KernelError(f"{self.prefix}: a layer without keys and values of its own only reads its cache slot")
+        y = self.in_linear(x)
+        write = kv.writes and not self.shared_kv
+        cos, sin = self.position.tables(y.device) if hasattr(self.position, "tables") else (None, None)
+        K.qk_encode_cache(y, batch.positions, self.num_heads, 0 if self.shared_kv else self.num_kv_heads, self.head_dim,
+                          self.value_dim, cos, sin, getattr(self.position, "pairing", "half") == "interleaved",
+                          self.norm_eps, kv.k_cache if write else None, kv.v_cache if write else None,
+                          kv.slot_mapping if write else None, q_weight=self.q_weight, k_weight=self.k_weight)
+        heads = torch.empty((y.shape[0], self.num_heads * self.value_dim), dtype=y.dtype, device=y.device)
+        attn_ops.paged_attention(y, heads, kv, batch, self.num_heads, self.num_kv_heads, self.head_dim, self.scale,
+                                 self.window, keep_first=self.keep_first, value_dim=self.value_dim, chunk=self.chunk)
+        return self.o(heads)

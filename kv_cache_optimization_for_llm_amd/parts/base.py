@@ -181,6 +181,16 @@ class NormedRows:
 
 
 @dataclass
+class StreamCopy:
+    """The residual stream as ``hidden`` holds it right now, once more in the type the products read
+    (a 32-bit stream of a bfloat16 model, rounded).  A block whose branches read the stream itself
+    hands it on in place of a pending branch output, so that the next block need not round the stream
+    again; whoever wants a pending output treats it as none."""
+
+    rows: torch.Tensor
+
+
+@dataclass
 class BranchTail:
     """What is to happen to a branch's output: it is added to ``hidden`` (the residual stream, in
     place) and the sum is handed to ``norm``, the norm that reads the stream next.  A mixer or
@@ -229,6 +239,11 @@ class Norm(Part):
         """``(weight, width, eps)`` if a product's epilogue may prepare this norm as
         :class:`NormedRows` (it must be ``x * rsqrt(mean(x^2) + eps) * weight``), else ``None``."""
         return None
+
+    def into_stream(self, stream: torch.Tensor, y: torch.Tensor, copy: Optional[torch.Tensor] = None) -> None:
+        """``stream += norm(y)`` in place, for arrangements that norm a branch's OUTPUT; ``copy``
+        receives the new stream in another type.  Norms that cannot be used this way do not have it."""
+        raise NotImplementedError(f"{type(self).__name__} cannot norm a branch output into the stream")
 
 
 class PositionEncoding(Part):

@@ -11,8 +11,10 @@ from typing import Optional
 
 import torch
 
-from ..config.registry import BLOCKS
-from .base import Block, BranchTail, MixerContext, Norm, NormedRows, PendingSum
+from ..config.registry import BLOCKS, LAYER_INPUTS
+from ..models.spec import PartSpec
+from ..ops import kernels as K
+from .base import Block, BranchTail, MixerContext, Norm, NormedRows, PendingSum, StreamCopy
 
 
 @BLOCKS.register("pre_norm")
@@ -95,3 +97,63 @@ class ParallelBlock(Block):
         if self.residual_mult != 1.0:
             return hidden, PendingSum(out, self.residual_mult)
         return hidden, out if self.has_ffn else a
+
+
+@BLOCKS.register("post_norm")
+class PostNormBlock(Block):
+    """The norm stands on every branch's OUTPUT: ``h += norm_m(mixer(h)); h += norm_f(ffn(h))``; the
+    branches read the stream itself.  ``layer_input`` (a :class:`~..models.spec.PartSpec` of the
+    ``LAYER_INPUTS`` registry) names a third branch that runs last and brings something from outside
+    the layer - the token's own row of a table - under a norm of its own: ``h += norm_i(input(h))``.
+    A layer without a feed-forward (``"none"``) names only the ``"mixer"`` norm.
+
+    Every sum and every norm is one pass (``ops.kernels.norm_into_stream``): it reads the branch's
+    output, norms it, adds it to the stream in the stream's own type, and - where the stream is kept in
+    32-bit under bfloat16 products - writes the rounded copy that the next branch reads, which is
+    handed on to the next block as :class:`~.base.StreamCopy`."""
+
+    graph_safe = True
+    NORM_NAMES = ("mixer", "feed_forward")
+
+    def __init__(self, mixer, feed_forward, norms, *, layer_input: Optional[PartSpec] = None):
+        self.has_ffn = not getattr(feed_forward, "absent", False)
+        if not self.has_ffn:
+            self.NORM_NAMES = ("mixer",)
+        super().__init__(mixer, feed_forward, norms)
+        self.layer_input = None
+        if layer_input is not None:
+            self.layer_input = LAYER_INPUTS.get(layer_input.kind)(**layer_input.params)
+
+    def parts(self):
+        return (*super().parts(), *((self.layer_input,) if self.layer_input is not None else ()))
+
+    def first_norm(self) -> Optional[Norm]:
+        return None
+
+    def _products_dtype(self) -> torch.dtype:
+        return self.norms["mixer"].weight.dtype     # vectors take the engine's compute type, like the matrices
+
+    def _into_stream(self, hidden, y, norm):
+        """``hidden += norm(y)``; returns the stream as the next branch reads it."""
+        if hidden.dtype == self._products_dtype():
+            norm.into_stream(hidden, y)
+            return hidden
+        copy = torch.empty(hidden.shape, dtype=self._products_dtype(), device=hidden.device)
+        norm.into_stream(hidden, y, copy)
+        return copy
+
+    def forward(self, hidden: torch.Tensor, delta, ctx: MixerContext, next_norm: Optional[Norm] = None):
+        if isinstance(delta, StreamCopy):
+            h = delta.rows
+        elif delta is not None:
+            raise TypeError("this arrangement takes the stream as it is, without pending branch outputs")
+        elif hidden.dtype == self._products_dtype():
+            h = hidden
+        else:
+            h = K.cast(hidden, torch.empty(hidden.shape, dtype=self._products_dtype(), device=hidden.device))
+        h = self._into_stream(hidden, self.mixer.forward(h, ctx), self.norms["mixer"])
+        if self.has_ffn:
+            h = self._into_stream(hidden, self.feed_forward.forward(h, ctx), self.norms["feed_forward"])
+        if self.layer_input is not None:
+            h = self._into_stream(hidden, self.layer_input.forward(h, ctx), self.layer_input)
+        return hidden, (StreamCopy(h) if h is not hidden else None)

@@ -5,6 +5,12 @@ Router: ``scores = softmax(W_router x)`` in fp32 over all router outputs.  The `
 the largest ``scores + correction`` (a stored vector that shifts the choice but not the weights)
 are chosen; their weights are the plain scores (``renormalise``: divided by their sum).  The last
 ``identity`` router outputs stand for experts that return their input: they have no tensors.
+``router_bias``: a stored vector added to the logits themselves; ``softmax_over="chosen"``: the
+largest logits are chosen and the weights are the softmax over the chosen logits alone.
+``gated``: an expert is ``W_down (act(W_gate x) * (W_up x))``; its gate and up matrices are stacked
+row by row in turns at load time, so that one product's epilogue has both halves of every output.
+``shared_intermediate``: one more expert of that width (its tensors behind ``shared.``) that every
+token uses with weight 1; it runs as an ordinary gated feed-forward and is added to the sum.
 
 Everything from the router's logits to the sum stays on the device (``csrc/moe.hip``): the chosen
 (token, choice) slots are sorted by expert into tiles of 16 rows, one kernel runs the first
@@ -34,10 +40,16 @@ class RoutedExperts(FeedForward):
 
     def __init__(self, prefix: str, *, hidden_size: int, intermediate_size: int, experts: int, top: int,
                  identity: int = 0, activation: str = "gelu", correction: bool = True, renormalise: bool = False,
-                 tensor_names: Optional[Dict[str, str]] = None):
-        """``tensor_names`` maps ``router``, ``correction``, ``up``, ``down`` to names behind ``prefix``;
-        the experts' names hold ``{e}`` for the expert's number."""
+                 gated: bool = False, router_bias: bool = False, softmax_over: str = "all",
+                 shared_intermediate: int = 0, tensor_names: Optional[Dict[str, str]] = None):
+        """``tensor_names`` maps ``router``, ``router_bias``, ``correction``, ``gate``, ``up``, ``down`` and
+        ``shared`` (a prefix) to names behind ``prefix``; the experts' names hold ``{e}`` for the expert's
+        number."""
         super().__init__(prefix)
+        if softmax_over not in ("all", "chosen"):
+            raise ValueError(f"{prefix}: softmax_over {softmax_over!r} is neither 'all' nor 'chosen'")
+        self.gated, self.has_router_bias, self.over_chosen = bool(gated), bool(router_bias), softmax_over == "chosen"
+        self.shared_intermediate = int(shared_intermediate)
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
         self.experts, self.top, self.identity = int(experts), int(top), int(identity)
         if self.experts < 0 or self.identity < 0 or not 0 < self.top <= self.experts + self.identity:
@@ -45,40 +57,68 @@ class RoutedExperts(FeedForward):
         if activation not in K.EXPERT_ACTIVATIONS:
             raise ValueError(f"activation {activation!r} is not one of {sorted(K.EXPERT_ACTIVATIONS)}")
         self.activation, self.has_correction, self.renormalise = activation, bool(correction), bool(renormalise)
-        names = dict(router="router", correction="correction", up="e{e}.up", down="e{e}.down")
+        names = dict(router="router", router_bias="router.b", correction="correction", gate="e{e}.gate", up="e{e}.up",
+                     down="e{e}.down", shared="shared.")
         names.update(tensor_names or {})
         self.names = {key: prefix + name for key, name in names.items()}
         self.outputs = self.experts + self.identity
+        self.shared = None
+        if self.shared_intermediate > 0:
+            if activation not in K.ACTIVATIONS:
+                raise ValueError(f"{prefix}: the expert every token uses runs with one of {sorted(K.ACTIVATIONS)}")
+            from .mlp import SwiGLU
+            self.shared = SwiGLU(self.names["shared"], hidden_size=self.hidden_size,
+                                 intermediate_size=self.shared_intermediate, activation=activation,
+                                 tensor_names=dict(gate="gate", up="up", down="down"))
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         n, W, I = self.names, self.hidden_size, self.intermediate_size
         specs = {n["router"]: TensorSpec((self.outputs, W))}
         if self.has_correction:
             specs[n["correction"]] = TensorSpec((self.outputs,), init="zeros", role="vector")
+        if self.has_router_bias:
+            specs[n["router_bias"]] = TensorSpec((self.outputs,), init="zeros", role="vector")
         for e in range(self.experts):
+            if self.gated:
+                specs[n["gate"].format(e=e)] = TensorSpec((I, W))
             specs[n["up"].format(e=e)] = TensorSpec((I, W))
             specs[n["down"].format(e=e)] = TensorSpec((W, I))
+        if self.shared is not None:
+            specs.update(self.shared.tensor_specs())
         return specs
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         n = self.names
         self.router = tensors[n["router"]].contiguous()             # its logits are formed in 32-bit (ops.kernels.small_product_f32)
         self.correction = tensors[n["correction"]].float().contiguous() if self.has_correction else None
-        if self.experts:
+        self.router_bias = tensors[n["router_bias"]].float().contiguous() if self.has_router_bias else None
+        if self.shared is not None:
+            self.shared.load(tensors)
+        if self.experts and self.gated:
+            # rows 2 j and 2 j + 1 of an expert's first matrix: output j's gate row and its up row
+            ups = []
+            for e in range(self.experts):
+                g, u = tensors[n["gate"].format(e=e)], tensors[n["up"].format(e=e)]
+                ups.append(torch.stack([g, u], dim=1).reshape(2 * g.shape[0], g.shape[1]))
+            self.w_up = torch.stack(ups).contiguous()
+            self.w_down = torch.stack([tensors[n["down"].format(e=e)] for e in range(self.experts)]).contiguous()
+        elif self.experts:
             self.w_up = torch.stack([tensors[n["up"].format(e=e)] for e in range(self.experts)]).contiguous()
             self.w_down = torch.stack([tensors[n["down"].format(e=e)] for e in range(self.experts)]).contiguous()
         else:
             self.w_up = self.w_down = None
 
     def activation_elements(self) -> int:
-        return self.outputs + self.top * (2 * self.intermediate_size + 2 * self.hidden_size) + self.hidden_size
+        return self.outputs + self.top * (2 * self.intermediate_size + 2 * self.hidden_size) + self.hidden_size \
+            + (self.shared.activation_elements() + self.hidden_size if self.shared is not None else 0)
 
     def forward(self, x, ctx: MixerContext, tail=None):
         T, dev = x.shape[0], x.device
-        logits = K.small_product_f32(x, self.router, torch.empty((T, self.outputs), dtype=torch.float32, device=dev))
+        logits = K.small_product_f32(x, self.router, torch.empty((T, self.outputs), dtype=torch.float32, device=dev),
+                                     bias=self.router_bias)
         idx = torch.empty((T, self.top), dtype=torch.int32, device=dev)
         wgt = torch.empty((T, self.top), dtype=torch.float32, device=dev)
-        K.moe_route(logits, self.correction, self.top, idx, wgt, self.renormalise)
+        K.moe_route(logits, self.correction, self.top, idx, wgt, self.renormalise, over_chosen=self.over_chosen)
         if RoutedExperts.on_route is not None and not torch.cuda.is_current_stream_capturing():
             RoutedExperts.on_route(self, idx)
         slots = T * self.top
@@ -89,7 +129,9 @@ class RoutedExperts(FeedForward):
             tile_expert = torch.empty(tiles, dtype=torch.int32, device=dev)
             K.moe_align(idx, self.experts, sorted_slot, tile_expert)
             act = torch.empty((tiles * K.MOE_TILE, self.intermediate_size), dtype=x.dtype, device=dev)
-            K.moe_expert_rows(x, self.w_up, act, sorted_slot, tile_expert, self.top, activation=self.activation)
+            K.moe_expert_rows(x, self.w_up, act, sorted_slot, tile_expert, self.top, activation=self.activation,
+                              gated=self.gated)
             K.moe_expert_rows(act, self.w_down, rows, sorted_slot, tile_expert, self.top, slot_weight=wgt)
         out = torch.empty_like(x)
-        return K.moe_combine(x, rows, idx, wgt, self.experts, out)
+        extra = self.shared.forward(x, ctx) if self.shared is not None else None
+        return K.moe_combine(x, rows, idx, wgt, self.experts, out, extra=extra)

@@ -38,6 +38,9 @@ class RMSNorm(Norm):
     def activation_elements(self) -> int:
         return self.width
 
+    def into_stream(self, stream, y, copy=None) -> None:
+        K.norm_into_stream(stream, y, self.weight, self.eps, copy)
+
     def forward(self, x, out=None, delta=None, row_idx=None):
         if out is None:
             rows = x.shape[0] if row_idx is None else row_idx.shape[0]
@@ -102,6 +105,11 @@ class LayerNorm(Norm):
         out = self._out(x, row_idx) if out is None else out
         return K.layernorm(x, self.weight, self.eps, out, deltas=self._deltas(delta), row_idx=row_idx,
                            rms=not self.center, delta_scale=self._scale(delta))
+
+    def into_stream(self, stream, y, copy=None) -> None:
+        if self.center:
+            raise NotImplementedError("only the form without the mean taken off norms a branch output into the stream")
+        K.norm_into_stream(stream, y, self.weight, self.eps, copy)
 
     def forward_pair(self, twin: "LayerNorm", x, delta=None):
         if twin.width != self.width or twin.eps != self.eps or twin.weight.dtype != self.weight.dtype \

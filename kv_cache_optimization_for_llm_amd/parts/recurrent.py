@@ -13,7 +13,12 @@ order of every sum depends on the sizes alone.
 * :class:`GatedDeltaRule` (``"gated_delta_rule"``): ``S <- g S; u = beta (v - S^T k); S <- S + k u^T;
   o = S^T q`` with one decay ``g = exp(-exp(A_log) softplus(a + dt_bias))`` and one step size
   ``beta = sigmoid(b)`` per head, unit-norm q and k, and a short causal convolution with silu on
-  q, k and v whose last inputs are part of the state.
+  q, k and v whose last inputs are part of the state.  ``decay="channel"``: the decay has one value
+  per head and key channel (a low-rank projection with a bias per channel and a rate per head) and
+  multiplies the rows of ``S`` one by one; ``gate_rank``: the output gate is a low-rank projection.
+* :class:`LightningAttention` (``"lightning_attention"``): ``S_t = decay_h S_(t-1) + k_t v_t^T``,
+  ``o_t = S_t^T q_t`` with one fixed decay a head, silu on q, k and v, and ONE norm over all heads'
+  read-outs together.
 """
 from __future__ import annotations
 
@@ -112,12 +117,26 @@ class GatedDeltaRule(ProjectedMixer):
 
     def __init__(self, prefix: str, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  value_dim: int, conv_taps: int, norm_eps: float, unit_eps: float = 1e-6,
+                 decay: str = "head", decay_rank: Optional[int] = None, gate: str = "silu",
+                 gate_rank: Optional[int] = None, low_rank_gate: bool = False,
                  tensor_names: Optional[Dict[str, str]] = None):
         """``num_kv_heads`` query/key heads serve ``num_heads`` value heads (head h uses q/k head
         ``h // (num_heads / num_kv_heads)``).  ``conv_taps``: length of the causal convolution on q, k, v
-        (1: none but the silu).  ``tensor_names`` maps ``q k v q_conv k_conv v_conv beta decay A_log dt_bias
-        g norm o`` to names behind ``prefix``."""
+        (1: none but the silu).  ``decay``: ``"head"`` - one decay a head, ``exp(-exp(A_log_h) softplus(W_a x +
+        dt_bias_h))`` - or ``"channel"`` - one per head and key channel, ``exp(-exp(A_log_h) softplus(W_a2 (W_a1
+        x) + dt_bias))`` with ``dt_bias`` of ``heads * head_dim`` values and the second product in 32-bit
+        (``decay_rank``: the inner size, ``None`` takes it from the stored tensors).  ``gate``: the activation
+        of the output gate (``"silu"`` or ``"sigmoid"``); ``low_rank_gate``: the gate is ``W_g2 (W_g1 x)``
+        (``gate_rank`` its inner size, ``None`` from the stored tensors).  ``tensor_names`` maps ``q k v q_conv
+        k_conv v_conv beta decay A_log dt_bias g norm o`` - and ``a1 a2 g1 g2`` - to names behind ``prefix``."""
         super().__init__(prefix)
+        if decay not in ("head", "channel"):
+            raise ValueError(f"{prefix}: decay {decay!r} is neither 'head' nor 'channel'")
+        if gate not in K.HEAD_GATES:
+            raise ValueError(f"{prefix}: gate {gate!r} is not one of {sorted(K.HEAD_GATES)}")
+        self.channel_decay, self.gate, self.low_rank_gate = decay == "channel", gate, bool(low_rank_gate)
+        self.decay_rank = None if decay_rank is None else int(decay_rank)
+        self.gate_rank = None if gate_rank is None else int(gate_rank)
         if num_heads % num_kv_heads:
             raise ValueError(f"{prefix}: {num_heads} heads is not a multiple of {num_kv_heads} key heads")
         if not 1 <= conv_taps <= 17:
@@ -128,31 +147,61 @@ class GatedDeltaRule(ProjectedMixer):
         self.inner_width = self.num_heads * self.value_dim
         self.conv_channels = 2 * self.num_kv_heads * self.head_dim + self.inner_width
         self.names = _names(dict(q="q", k="k", v="v", q_conv="q.conv", k_conv="k.conv", v_conv="v.conv", beta="b",
-                                 decay="a", A_log="A_log", dt_bias="dt_bias", g="g", norm="norm", o="o"),
+                                 decay="a", A_log="A_log", dt_bias="dt_bias", g="g", norm="norm", o="o",
+                                 a1="a1", a2="a2", g1="g1", g2="g2"),
                             tensor_names, prefix)
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         n, W, gd, hv, H, taps = self.names, self.hidden_size, self.num_kv_heads * self.head_dim, self.inner_width, \
             self.num_heads, self.conv_taps
-        return {
+        specs = {
             n["q"]: TensorSpec((gd, W)), n["k"]: TensorSpec((gd, W)), n["v"]: TensorSpec((hv, W)),
             n["q_conv"]: TensorSpec((gd, taps), init="norm", role="vector"),
             n["k_conv"]: TensorSpec((gd, taps), init="norm", role="vector"),
             n["v_conv"]: TensorSpec((hv, taps), init="norm", role="vector"),
-            n["beta"]: TensorSpec((H, W)), n["decay"]: TensorSpec((H, W)),
+            n["beta"]: TensorSpec((H, W)),
             n["A_log"]: TensorSpec((H,), init="zeros", role="vector"),
-            n["dt_bias"]: TensorSpec((H,), init="zeros", role="vector"),
-            n["g"]: TensorSpec((hv, W)), n["norm"]: TensorSpec((self.value_dim,), init="norm", role="vector"),
+            n["norm"]: TensorSpec((self.value_dim,), init="norm", role="vector"),
             n["o"]: TensorSpec((W, hv)),
         }
+        if self.channel_decay:
+            specs[n["a1"]] = TensorSpec((self.decay_rank, W))
+            specs[n["a2"]] = TensorSpec((H * self.head_dim, self.decay_rank))
+            specs[n["dt_bias"]] = TensorSpec((H * self.head_dim,), init="zeros", role="vector")
+        else:
+            specs[n["decay"]] = TensorSpec((H, W))
+            specs[n["dt_bias"]] = TensorSpec((H,), init="zeros", role="vector")
+        if self.low_rank_gate:
+            specs[n["g1"]] = TensorSpec((self.gate_rank, W))
+            specs[n["g2"]] = TensorSpec((hv, self.gate_rank))
+        else:
+            specs[n["g"]] = TensorSpec((hv, W))
+        return specs
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
-        t = {key: tensors[name] for key, name in self.names.items()}
-        self._w_in = torch.cat([t["q"], t["k"], t["v"], t["beta"], t["decay"], t["g"]], dim=0).contiguous()
+        t = {key: tensors[name] for key, name in self.names.items() if name in tensors}
+        # the joined projection's rows: q, k, v, beta, then what makes the decay, then what makes the gate
+        decay_rows = t["a1"] if self.channel_decay else t["decay"]
+        gate_rows = t["g1"] if self.low_rank_gate else t["g"]
+        if self.channel_decay and t["a1"].shape[0] != t["a2"].shape[1]:
+            raise ValueError(f"{self.prefix}: the decay's two matrices do not fit each other: "
+                             f"{tuple(t['a1'].shape)} and {tuple(t['a2'].shape)}")
+        if self.low_rank_gate and t["g1"].shape[0] != t["g2"].shape[1]:
+            raise ValueError(f"{self.prefix}: the gate's two matrices do not fit each other: "
+                             f"{tuple(t['g1'].shape)} and {tuple(t['g2'].shape)}")
+        self._w_in = torch.cat([t["q"], t["k"], t["v"], t["beta"], decay_rows, gate_rows], dim=0).contiguous()
         self._w_out = t["o"]
         self.beta_off = self.conv_channels
         self.decay_off = self.beta_off + self.num_heads
-        self.g_off = self.decay_off + self.num_heads
+        self.decay_cols = int(decay_rows.shape[0])
+        self.g_off = self.decay_off + self.decay_cols
+        self.gate_cols = int(gate_rows.shape[0])
+        # decays per channel are formed in 32-bit: the low-rank projection's second matrix multiplies in fp32
+        self.a2 = t["a2"].contiguous() if self.channel_decay else None
+        self.g2 = None
+        if self.low_rank_gate:
+            from .linear import Linear
+            self.g2 = Linear(t["g2"])
         self.conv_weight = torch.cat([t["q_conv"], t["k_conv"], t["v_conv"]], dim=0).float().contiguous()
         self.a_log, self.dt_bias = t["A_log"].float().contiguous(), t["dt_bias"].float().contiguous()
         self.norm_weight = t["norm"].float().contiguous()
@@ -178,8 +227,87 @@ class GatedDeltaRule(ProjectedMixer):
         K.causal_conv_act(y, col0, self.conv_weight, qkv, ctx.state, state_off + s_elems, batch.entry_q_start,
                           batch.entry_seat, batch.max_q_len)
         o = torch.empty((T, self.inner_width), dtype=torch.float32, device=y.device)
-        K.gated_delta_rule(qkv, y, col0 + self.beta_off, col0 + self.decay_off, self.a_log, self.dt_bias, o, ctx.state,
-                           state_off, batch.entry_q_start, batch.entry_seat, self.num_heads, self.num_kv_heads,
-                           self.head_dim, self.value_dim, self.unit_eps)
-        K.head_norm_gate(o, self.norm_weight, self.norm_eps, y, col0 + self.g_off, out, out_col0, self.num_heads,
-                         self.value_dim, "silu", mul)
+        if self.channel_decay:
+            # bias, softplus, the head's rate and the exponential in the second product's epilogue
+            d0 = col0 + self.decay_off
+            g = K.small_product_f32(y[:, d0:d0 + self.decay_cols], self.a2,
+                                    torch.empty((T, self.num_heads * self.head_dim), dtype=torch.float32, device=y.device),
+                                    bias=self.dt_bias, rate_log=self.a_log)
+            K.gated_delta_rule(qkv, y, col0 + self.beta_off, 0, None, None, o, ctx.state, state_off,
+                               batch.entry_q_start, batch.entry_seat, self.num_heads, self.num_kv_heads,
+                               self.head_dim, self.value_dim, self.unit_eps, channel_decay=g)
+        else:
+            K.gated_delta_rule(qkv, y, col0 + self.beta_off, col0 + self.decay_off, self.a_log, self.dt_bias, o,
+                               ctx.state, state_off, batch.entry_q_start, batch.entry_seat, self.num_heads,
+                               self.num_kv_heads, self.head_dim, self.value_dim, self.unit_eps)
+        if self.low_rank_gate:
+            g0 = col0 + self.g_off
+            gate, gate_off = self.g2(y[:, g0:g0 + self.gate_cols].contiguous()), 0
+        else:
+            gate, gate_off = y, col0 + self.g_off
+        K.head_norm_gate(o, self.norm_weight, self.norm_eps, gate, gate_off, out, out_col0, self.num_heads,
+                         self.value_dim, self.gate, mul)
+
+
+@MIXERS.register("lightning_attention")
+class LightningAttention(ProjectedMixer):
+    """Linear attention with one fixed decay a head: ``S_t = decay_h S_(t-1) + k_t v_t^T``, ``o_t = S_t^T
+    (query_scale q_t)`` where q, k and v are the ``activation`` (silu) of their projections.  The heads'
+    read-outs are normed TOGETHER (one RMS norm over ``heads * value_dim`` elements with a weight of
+    that size), gated element by element with ``gate(W_g x)`` and projected.  The decays are
+    constants of the model, not tensors.  State: ``S`` of every head, fp32."""
+
+    graph_safe = True
+
+    def __init__(self, prefix: str, *, hidden_size: int, num_heads: int, head_dim: int, value_dim: int, decay,
+                 norm_eps: float, query_scale: float = 1.0, activation: Optional[str] = "silu", gate: str = "sigmoid",
+                 tensor_names: Optional[Dict[str, str]] = None):
+        """``decay``: one number a head.  ``tensor_names`` maps ``q k v g o norm`` to names behind ``prefix``."""
+        super().__init__(prefix)
+        self.hidden_size, self.num_heads, self.head_dim, self.value_dim = int(hidden_size), int(num_heads), int(head_dim), int(value_dim)
+        self.decay = tuple(float(a) for a in decay)
+        if len(self.decay) != self.num_heads:
+            raise ValueError(f"{prefix}: {len(self.decay)} decays for {self.num_heads} heads")
+        if gate not in K.HEAD_GATES:
+            raise ValueError(f"{prefix}: gate {gate!r} is not one of {sorted(K.HEAD_GATES)}")
+        self.norm_eps, self.query_scale, self.activation, self.gate = float(norm_eps), float(query_scale), activation, gate
+        self.inner_width = self.num_heads * self.value_dim
+        self.names = _names(dict(q="q", k="k", v="v", g="g", o="o", norm="norm"), tensor_names, prefix)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        n, W, hd, hv = self.names, self.hidden_size, self.num_heads * self.head_dim, self.inner_width
+        return {n["q"]: TensorSpec((hd, W)), n["k"]: TensorSpec((hd, W)), n["v"]: TensorSpec((hv, W)),
+                n["g"]: TensorSpec((hv, W)), n["o"]: TensorSpec((W, hv)),
+                n["norm"]: TensorSpec((hv,), init="norm", role="vector")}
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        t = {key: tensors[name] for key, name in self.names.items()}
+        self._w_in = torch.cat([t["q"], t["k"], t["v"], t["g"]], dim=0).contiguous()
+        self._w_out = t["o"]
+        hd, hv = self.num_heads * self.head_dim, self.inner_width
+        self.q_off, self.k_off, self.v_off, self.g_off = 0, hd, 2 * hd, 2 * hd + hv
+        self.norm_weight = t["norm"].float().contiguous()
+        self.head_decay = torch.tensor(self.decay, dtype=torch.float32, device=self._w_in.device)
+        self.load_projections()
+
+    def input_weight(self) -> torch.Tensor:
+        return self._w_in
+
+    def output_weight(self) -> torch.Tensor:
+        return self._w_out
+
+    def state_elements(self) -> int:
+        return self.num_heads * self.head_dim * self.value_dim
+
+    def activation_elements(self) -> int:
+        return 2 * self.num_heads * self.head_dim + 5 * self.inner_width + self.hidden_size
+
+    def forward_inner(self, y, col0, ctx: MixerContext, state_off, out, out_col0, mul) -> None:
+        batch, T = ctx.batch, y.shape[0]
+        o = torch.empty((T, self.inner_width), dtype=torch.float32, device=y.device)
+        K.gated_linear_attention(y, col0 + self.q_off, col0 + self.k_off, col0 + self.v_off, None, self.query_scale, o,
+                                 ctx.state, state_off, batch.entry_q_start, batch.entry_seat, self.num_heads,
+                                 self.head_dim, self.value_dim, head_decay=self.head_decay, activation=self.activation)
+        # one norm over all the heads' read-outs: a single "head" as wide as the row
+        K.head_norm_gate(o, self.norm_weight, self.norm_eps, y, col0 + self.g_off, out, out_col0, 1, self.inner_width,
+                         self.gate, mul)
