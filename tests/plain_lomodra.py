@@ -146,12 +146,19 @@ def router_logits(W, p: str, h):
     return h @ W[p + "router"].T + W[p + "router.b"]
 
 
-def mixture(W, p: str, mlp: dict, h, rounded=_same, choices=None):
+def mixture(W, p: str, mlp: dict, h, rounded=_same, choices=None, margin_out=None):
     """The ``top`` experts with the largest logits, weighted by the softmax over those logits alone,
-    plus the expert every token uses.  ``choices`` [T, top] overrides the router's own choice."""
+    plus the expert every token uses.  ``choices`` [T, top] overrides the router's own choice;
+    ``margin_out`` (a list) receives (own choice, logit gap between the last chosen and the first
+    left-out expert)."""
     E, top = mlp["router"]["experts"], mlp["router"]["top"]
     z = router_logits(W, p, h)
-    idx = torch.topk(z, top, dim=-1).indices if choices is None else choices.long()
+    own = torch.topk(z, top, dim=-1).indices
+    if margin_out is not None:
+        ordered = torch.sort(z, dim=-1, descending=True).values
+        gap = ordered[:, top - 1] - ordered[:, top] if top < E else torch.full((h.shape[0],), float("inf"), dtype=F)
+        margin_out.append((own, gap))
+    idx = own if choices is None else choices.long()
     wgt = torch.softmax(torch.gather(z, 1, idx), dim=-1)
     out = torch.zeros_like(h)
     for e in range(E):
@@ -176,10 +183,16 @@ def token_side(W, layer: int, dim: int, x, h, tokens, eps: float, rounded=_same)
 
 
 # ---- the model ----------------------------------------------------------------------------------
-def forward(cfg: dict, W: Dict[str, torch.Tensor], tokens: List[int], rounded=_same, choices=None,
-            layer_outputs: Optional[list] = None):
-    """Logits [T, vocab] of one whole sequence.  ``W`` holds float64 tensors by name.  ``choices`` maps
-    a layer index to the experts [T, top] its tokens are sent to (else the router decides)."""
+def to_f64(state: Dict[str, torch.Tensor]) -> Dict[str, torch.Tensor]:
+    return {k: v.to(F) for k, v in state.items()}
+
+
+def forward(cfg: dict, W: Dict[str, torch.Tensor], tokens: List[int], rounded=_same, forced=None,
+            layer_outputs: Optional[list] = None, margins: Optional[dict] = None):
+    """Logits [T, vocab] of one whole sequence.  ``W`` holds float64 tensors by name.  ``forced`` maps
+    a layer index to the experts [T, top] its tokens are sent to (else the router decides);
+    ``margins`` receives per layer (the router's own choice, its margin)."""
+    choices = forced
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     eps = float(cfg["norm"]["eps"])
     x = W["embed"][tokens].clone()
@@ -197,7 +210,10 @@ def forward(cfg: dict, W: Dict[str, torch.Tensor], tokens: List[int], rounded=_s
             y = attention(W, p, m, h, eps, kept[i if m.get("kv_from") is None else m["kv_from"]], rounded)
         x = x + rms_norm(y, W[f"l{i}.norm1"], eps)
         if layer.get("mlp") is not None:
-            y = mixture(W, f"l{i}.mlp.", layer["mlp"], rounded(x), rounded, None if choices is None else choices.get(i))
+            got = [] if margins is not None else None
+            y = mixture(W, f"l{i}.mlp.", layer["mlp"], rounded(x), rounded, None if choices is None else choices.get(i), got)
+            if got:
+                margins[i] = got[0]
             x = x + rms_norm(rounded(y), W[f"l{i}.norm2"], eps)
         if cfg.get("token_side") is not None:
             x = token_side(W, i, int(cfg["token_side"]["dim"]), x, rounded(x), tokens, eps, rounded)
