@@ -1,0 +1,95 @@
+"""Lomodra models drawn at random - layer order, widths, head counts and sizes, chunk sizes, layers that
+take an earlier layer's keys and values, taps, ranks, routers, constants, missing feed-forwards and
+token inputs - stepped through a random mixed schedule on a small pool and compared with the plain
+implementation, in both number formats; and, with graphs, through the trace runner's own options."""
+import numpy as np
+import pytest
+
+import lomodra_util as U
+import replay_util as R
+from kv_cache_optimization_for_llm_amd.engine.engine import Engine, EngineOptions
+
+pytestmark = pytest.mark.gpu
+
+
+def random_config(seed: int) -> dict:
+    rng = np.random.default_rng(seed)
+    pick = lambda *xs: xs[int(rng.integers(len(xs)))]
+    width = pick(64, 72, 96, 100, 128, 160, 256, 320)
+
+    def mlp():
+        if rng.random() < 0.2:
+            return None
+        experts = pick(1, 2, 3, 4, 7, 8, 9, 16)
+        return U.moe(experts, int(rng.integers(1, experts + 1)), pick(16, 24, 32, 64, 96),
+                     shared=pick(None, 8, 32, 96))
+
+    layers, owners = [], []            # owners: attention layers with keys and values of their own
+    for i in range(int(rng.integers(2, 7))):
+        kind = pick("attention", "attention", "lightning", "channel_delta")
+        if kind == "lightning":
+            heads = pick(1, 2, 3, 4, 5)
+            decay = [float(pick(1.0, 0.999, 0.97, 0.9, 0.6, 0.3)) for _ in range(heads)]
+            layers.append(U.lightning_layer(heads, pick(8, 16, 24, 48, 64, 128, 136), pick(4, 8, 20, 32, 64), decay, mlp()))
+        elif kind == "channel_delta":
+            kv = pick(1, 2, 3)
+            dim = pick(8, 16, 32, 40, 64, 128, 144)
+            layers.append(U.delta_layer(kv * pick(1, 2, 3), kv, dim, pick(dim, 8, 24, 64), pick(1, 2, 4, 7),
+                                        pick(1, 3, 8, 24), pick(2, 5, 16, 24), mlp()))
+        else:
+            chunk = pick(None, 1, 5, 16, 31, 32, 64, 100)
+            if owners and rng.random() < 0.4:
+                j = owners[int(rng.integers(len(owners)))]
+                m = layers[j]["mixer"]
+                layers.append(U.attention_layer(m["heads"], m["kv_heads"], m["dim"], m["vdim"], pick(0.08, 0.125, 0.3),
+                                                chunk, kv_from=j, mlp=mlp()))
+            else:
+                kv, dim = pick(1, 2, 3), pick(16, 20, 32, 48, 64, 96, 128)
+                owners.append(len(layers))
+                layers.append(U.attention_layer(kv * pick(1, 2, 4), kv, dim, pick(dim, 16, 32, 64), pick(0.08, 0.125, 0.3),
+                                                chunk, mlp=mlp()))
+    cfg = {"architecture": "Lomodra", "vocab": pick(64, 101, 256, 333, 448), "width": width,
+           "norm": {"eps": pick(0.02, 0.05, 0.1)}, "layers": layers}
+    if rng.random() < 0.8:
+        cfg["logit_softcap"] = float(pick(5.0, 15.0, 30.0))
+    if rng.random() < 0.8:
+        cfg["token_side"] = {"dim": pick(1, 4, 12, 16, 32)}
+    return cfg
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(16))
+def test_random_models_under_random_schedules(seed, dtype, tmp_path, gpu):
+    cfg = random_config(3000 + seed)
+    folder, state = U.write_model(str(tmp_path / "m"), cfg, seed, gain=0.8)
+    rng = np.random.default_rng(seed)
+    lengths = [int(n) for n in rng.integers(1, 140, size=7)]
+    reqs = {f"q{i}": U.prompt(cfg, n, 13 * i + seed) for i, n in enumerate(lengths)}
+    steps = R.mixed(reqs, seed=seed, max_live=4, chunk_sizes=(2, 3, 7, 16, 40))
+    eng = Engine(folder, EngineOptions(dtype=dtype, page_size=16, cache_tokens=R.max_live_tokens(steps, unit=16),
+                                       max_seqs=4, max_seq_len=160, max_batch_tokens=1024, use_graphs=False))
+    rows, routes = U.run_steps(eng, steps, cfg)
+    assert len(rows) == sum(lengths)
+    U.assert_rows(rows, U.expected_rows(cfg, state, reqs, routes, dtype), dtype, f"model {cfg}")
+    eng.cache.check()
+    assert eng.cache.free_seats == 4 and all(g.free_pages() == g.num_pages for g in eng.cache.groups)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_models_with_graphs_equal_eager_steps(seed, tmp_path, gpu):
+    """The bf16 engine as it serves (decode steps and portion steps whose shape comes back from HIP
+    graphs) gives what its eager steps give, for models drawn at random."""
+    cfg = random_config(3100 + seed)
+    folder, state = U.write_model(str(tmp_path / "m"), cfg, seed, gain=0.8)
+    reqs = {f"g{i}": U.prompt(cfg, n, 5 * i + seed) for i, n in enumerate([70, 33, 101])}
+    steps = R.tail_decoded(reqs, tail=24) + R.tail_decoded({k + "x": v for k, v in reqs.items()}, tail=24)
+    for i, st in enumerate(steps):
+        st["step"] = i
+    opts = dict(dtype="bfloat16", page_size=16, cache_tokens=512, max_seqs=4, max_seq_len=160, max_batch_tokens=1024)
+    eager = U.run_steps(Engine(folder, EngineOptions(use_graphs=False, **opts)), steps)
+    eng = Engine(folder, EngineOptions(use_graphs=True, **opts))
+    assert eng.graphs is not None, "every part of the model can be captured"
+    replayed = U.run_steps(eng, steps)
+    assert eng.graphs.replays > 0
+    for key in eager:
+        np.testing.assert_array_equal(eager[key], replayed[key], err_msg=str(key))
