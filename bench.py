@@ -15,7 +15,7 @@ tokens, each with its step time, bytes and fraction of the HBM peak, and the ser
 (``kclass_...``; ``--no-kernel-classes`` leaves them out) and, for the serving runs, pages reused,
 preemptions and fragmentation failures.
 
-    python bench.py --design gadopel|radilix [--layers 8]
+    python bench.py --design gadopel|radilix|lomodra [--layers 8]
 
 is another measurement with a JSON line of its own (the default run above is untouched): prefill
 and decode throughput of a Gadopel model at layer sizes of a served model (random weights), beside
@@ -108,6 +108,31 @@ def radilix_config(layers: int, vocab: int, width: int = 2048) -> dict:
             "layers": [gla if i % 4 == 3 else side for i in range(layers)], "max_positions": 8192}
 
 
+# --design lomodra: layers of width W in runs of four - softmax attention inside chunks of 1,024 positions
+# (W / 64 heads of 64 over W / 256 kv heads, normed queries and keys), a delta rule with a decay per key
+# channel (W / 256 value heads of 128 over W / 512 query/key heads of 128, four taps, ranks of 64), lightning
+# attention (W / 128 heads of 64 x 128), and an attention layer that reads the first one's keys and values.
+# Every layer has 16 gated experts of width 3 W / 8 (three matrices: 1.125 W^2 weights an expert, against
+# the Radilix expert's W^2), 4 choices a token, one more expert of that width that every token uses, and a
+# token input of 64 columns.  Beside it run the closest design, Radilix (recurrences and routed experts
+# too), and the Llama model, both at the same width.
+def lomodra_config(layers: int, vocab: int, width: int = 2048) -> dict:
+    W = width
+    mlp = {"kind": "moe", "expert": {"ff": 3 * W // 8}, "router": {"experts": 16, "top": 4}, "shared": {"ff": 3 * W // 8}}
+    attn = {"heads": W // 64, "kv_heads": W // 256, "dim": 64, "vdim": 64, "scale": 0.125, "mask": {"size": 1024}}
+    kinds = [
+        lambda i: {"type": "attention", "mlp": mlp, "mixer": dict(attn)},
+        lambda i: {"type": "channel_delta", "mlp": mlp, "mixer": {"heads": W // 256, "kv_heads": W // 512, "dim": 128,
+                                                                   "vdim": 128, "conv": 4, "decay_rank": 64, "gate_rank": 64}},
+        lambda i: {"type": "lightning", "mlp": mlp, "mixer": {"heads": W // 128, "dim": 64, "vdim": 128,
+                                                               "decay": [1.0 - 2.0 ** -(3 + 5 * h / max(1, W // 128 - 1))
+                                                                         for h in range(W // 128)]}},
+        lambda i: {"type": "attention", "mlp": mlp, "mixer": dict(attn, kv_from=i - 3)},
+    ]
+    return {"architecture": "Lomodra", "vocab": vocab, "width": W, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+            "token_side": {"dim": 64}, "layers": [kinds[i % 4](i) for i in range(layers)], "max_positions": 8192}
+
+
 def design_comparison(args) -> int:
     import torch
     from kv_cache_optimization_for_llm_amd.engine.batch import StepEntry
@@ -118,15 +143,17 @@ def design_comparison(args) -> int:
     llama = dict(CONFIG_1B, num_hidden_layers=layers, vocab_size=vocab, tie_word_embeddings=False)
     design, width = args.design, args.width
     if width != 2048:
-        if design != "radilix" or width % 512 or not 512 <= width <= 8192:
-            print("--width: a multiple of 512 from 512 to 8192, for --design radilix")
+        if design not in ("radilix", "lomodra") or width % 512 or not 512 <= width <= 8192:
+            print("--width: a multiple of 512 from 512 to 8192, for --design radilix or lomodra")
             return 2
         llama.update(hidden_size=width, intermediate_size=4 * width, num_attention_heads=width // 64,
                      num_key_value_heads=width // 256)
-        made = radilix_config(layers, vocab, width)
+    if design == "lomodra":
+        configs = {design: lomodra_config(layers, vocab, width), "radilix": radilix_config(layers, vocab, width), "llama": llama}
+    elif design == "radilix":
+        configs = {design: radilix_config(layers, vocab, width), "llama": llama}
     else:
-        made = {"gadopel": gadopel_config, "radilix": radilix_config}[design](layers, vocab)
-    configs = {design: made, "llama": llama}
+        configs = {design: gadopel_config(layers, vocab), "llama": llama}
     shapes = [(8, 4096), (32, 2048)]            # (requests, context) of the decode runs
     gen = torch.Generator().manual_seed(0)
     out = {}
@@ -202,7 +229,7 @@ def design_comparison(args) -> int:
     print(json.dumps({"metric": f"{design}_decode_tokens_per_second", "value": out[design][f"decode_b{b}_c{c}_tok_s"],
                       "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
                       "higher_is_better": True, "dtype": "bf16", "data": "synthetic (random weights, seeded token ids)",
-                      "config": {"design": f"{design} beside llama", "layers": layers, "width": width, "ff": 4 * width,
+                      "config": {"design": f"{design} beside " + " and ".join(n for n in configs if n != design), "layers": layers, "width": width, "ff": 4 * width,
                                  "vocab": vocab, "decode_shapes": shapes, "prefill_tokens": PREFILL_TOKENS},
                       "designs": out}))
     return 0
@@ -210,10 +237,10 @@ def design_comparison(args) -> int:
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", choices=["gadopel", "radilix"], default=None,
+    ap.add_argument("--design", choices=["gadopel", "radilix", "lomodra"], default=None,
                     help="another measurement (its own JSON line): a model of this design at the layer sizes of a "
                          "served model beside a Llama model of equal size; the default run is left as it is")
-    ap.add_argument("--width", type=int, default=2048, help="--design radilix: the models' width (head counts and "
+    ap.add_argument("--width", type=int, default=2048, help="--design radilix or lomodra: the models' width (head counts and "
                     "feed-forward sizes scale with it)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
