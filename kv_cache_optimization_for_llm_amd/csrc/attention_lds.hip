@@ -76,21 +76,22 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, float *__restrict__ part
         tq[rt] = row_valid[rt] ? row / G : 0;
         head[rt] = kvh * G + (row_valid[rt] ? row % G : 0);
         my_pos[rt] = start_pos + tq[rt];
-        my_lo[rt] = (window > 0 && my_pos[rt] - window + 1 > 0) ? my_pos[rt] - window + 1 : 0;
+        my_lo[rt] = kva_first_visible_signed(my_pos[rt], window);
     }
     const int w_last = (wrow0 + 31 < M - 1) ? wrow0 + 31 : M - 1;
     // (uniform over the wavefront: said explicitly, since the division by G is done in the vector
     // ALU and the compiler then takes every test on these for a per-lane one)
     const int w_hi = __builtin_amdgcn_readfirstlane(start_pos + w_last / G);      // last key the wave sees
     const int w_first_pos = __builtin_amdgcn_readfirstlane(start_pos + wrow0 / G);
-    const int w_lo = (window > 0 && w_first_pos - window + 1 > 0) ? w_first_pos - window + 1 : 0;
+    const int w_lo = kva_first_visible_signed(w_first_pos, window);
+    const int w_hi_lo = kva_first_visible_signed(w_hi, window);      // where the window (or chunk) of the wave's last row starts
     const bool all_rows = wrow0 + 32 <= M;
 
     // ---- keys the workgroup visits
     const int g_last = (row0 + 127 < M - 1) ? row0 + 127 : M - 1;
     const int g_hi = __builtin_amdgcn_readfirstlane(start_pos + g_last / G);
     const int g_first_pos = __builtin_amdgcn_readfirstlane(start_pos + row0 / G);
-    const int g_lo = (window > 0 && g_first_pos - window + 1 > 0) ? g_first_pos - window + 1 : 0;
+    const int g_lo = kva_first_visible_signed(g_first_pos, window);
     int k_begin = g_lo & ~31;
     int k_end = g_hi + 1;
     if (splits > 1) {               // uniform over the workgroup; an empty range leaves m = -inf, l = 0
@@ -298,7 +299,7 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, float *__restrict__ part
     // Loads past the end are redirected inside fetch (never out of the mapped pages) and unused.
     auto compute = [&](const char *buf, int kstart) {
         if (wave_valid && kstart < k_end && kstart <= w_hi && kstart + 31 >= w_lo) {
-            const bool masked = window > 0 || kstart + 31 > w_first_pos || !all_rows;
+            const bool masked = kstart < w_hi_lo || kstart + 31 > w_first_pos || !all_rows;
             if (masked) compute_as(std::true_type{}, buf, kstart);
             else compute_as(std::false_type{}, buf, kstart);
         }
@@ -437,7 +438,7 @@ extern "C" int kva_attention_lds(void *out, float *part_o, float *part_ml, const
     KVA_REQUIRE(kva_attention_lds_supported(head_dim, page_size),
                 "attention_lds: head_dim %d with pages of %d keys is not supported (32/64/96/128, 16)", head_dim, page_size);
     KVA_REQUIRE(q_row_stride % 8 == 0 && q_row_stride >= num_q_heads * head_dim, "attention_lds: q row stride %d", q_row_stride);
-    KVA_REQUIRE(window >= 0 && scale > 0.f, "attention_lds: window must not be negative and the scale positive");
+    KVA_REQUIRE(scale > 0.f, "attention_lds: the scale must be positive");     // (window < 0: chunks of -window positions)
     KVA_REQUIRE(item_meta != nullptr || num_items == 0, "attention_lds: item records are needed");
     if (num_items == 0) return KVA_OK;
     const int groups = pair ? (num_items + 1) / 2 : num_items;

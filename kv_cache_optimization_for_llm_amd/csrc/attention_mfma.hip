@@ -130,7 +130,7 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
         tq[rt] = row_valid[rt] ? row / G : 0;
         head[rt] = kvh * G + (row_valid[rt] ? row % G : 0);
         my_pos[rt] = start_pos + tq[rt];
-        my_lo[rt] = (window > 0 && my_pos[rt] - window + 1 > 0) ? my_pos[rt] - window + 1 : 0;
+        my_lo[rt] = kva_first_visible_signed(my_pos[rt], window);
     }
 
     // keys any row of this item may see
@@ -139,7 +139,8 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
     // is done in the vector ALU and the compiler then takes every test on these for a per-lane one)
     const int item_hi = __builtin_amdgcn_readfirstlane(start_pos + last_row / G);                       // inclusive
     const int item_pos_lo = __builtin_amdgcn_readfirstlane(start_pos + row0 / G);
-    const int item_lo = (window > 0 && item_pos_lo - window + 1 > 0) ? item_pos_lo - window + 1 : 0;
+    const int item_lo = kva_first_visible_signed(item_pos_lo, window);
+    const int item_hi_lo = kva_first_visible_signed(item_hi, window);     // where the window (or chunk) of the item's last row starts
     int k_begin = item_lo & ~31;
     int k_end = item_hi + 1;                                            // exclusive
     if (splits > 1) {
@@ -474,7 +475,7 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
             }
         }
         // incl. redirected tiles and items whose last row tile is cut short
-        const bool masked = window > 0 || kstart + 31 > first_pos || !all_rows;
+        const bool masked = kstart < item_hi_lo || kstart + 31 > first_pos || !all_rows;
         if (masked) compute_block_as(std::true_type{}, f, kstart);
         else compute_block_as(std::false_type{}, f, kstart);
     };
@@ -802,7 +803,7 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
     KVA_REQUIRE(splits == waves || (part_o && part_ml), "attention_mfma: key ranges of several workgroups need a workspace");
     // without `out` the partial results (splits / waves a row) are left to the caller: no merge launch
     KVA_REQUIRE(out != nullptr || splits / waves > 1, "attention_mfma: no output");
-    KVA_REQUIRE(window >= 0, "attention_mfma: negative window");
+    // (window < 0: chunks of -window positions - a query sees the keys of its own chunk up to itself)
     KVA_REQUIRE(scale > 0.f, "attention_mfma: the score scale must be positive");
     KVA_REQUIRE(row_tiles == 1 || row_tiles == kva_attention_mfma_row_tiles(head_dim, 1),
                 "attention_mfma: %d row tiles per item is not what head_dim %d is built with", row_tiles, head_dim);

@@ -25,3 +25,9 @@ __host__ __device__ inline int kva_first_visible(int pos, int window, int chunk)
     if (chunk > 0) return pos - pos % chunk;
     return (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
 }
+
+// The same for kernels that take both masks in one number: `window` > 0 is a window of so many
+// positions, `window` < 0 stands for chunks of -window positions, 0 for every earlier key.
+__host__ __device__ inline int kva_first_visible_signed(int pos, int window) {
+    return window < 0 ? pos - pos % (-window) : ((window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0);
+}

@@ -247,10 +247,13 @@ latent_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_o, 
     for (int s = 0; s < splits; ++s) m = fmaxf(m, ml[2 * s]);
     float den = sinks ? __builtin_amdgcn_exp2f(sinks[row % heads] * LAT_LOG2E - m) : 0.f;
     for (int s = 0; s < splits; ++s) den += __builtin_amdgcn_exp2f(ml[2 * s] - m) * ml[2 * s + 1];
+    // (a range without a visible key - most of them under a window or chunks - has l = 0 and is not read;
+    // the order of the others stays, so the sum does not depend on how many empty ones lie between)
     for (int j = threadIdx.x; j < rank; j += blockDim.x) {
         float acc = 0.f;
         for (int s = 0; s < splits; ++s)
-            acc += __builtin_amdgcn_exp2f(ml[2 * s] - m) * part_o[(row * splits + s) * rank + j];
+            if (ml[2 * s + 1] != 0.f)
+                acc += __builtin_amdgcn_exp2f(ml[2 * s] - m) * part_o[(row * splits + s) * rank + j];
         out[row * rank + j].bits = float_to_bf16_bits(acc / den);
     }
 }

@@ -728,14 +728,47 @@ head_norm_gate_kernel(void *__restrict__ out, int out_dtype, int out_stride, int
     }
 }
 
+// Few wide heads (one norm over a whole row, say): the workgroup takes the heads one after the other,
+// all its wavefronts on each; the sum of squares is taken in a fixed order.
+__global__ void __launch_bounds__(256)
+head_norm_gate_wide_kernel(void *__restrict__ out, int out_dtype, int out_stride, int out_off, const void *__restrict__ x,
+                           int x_dtype, const float *__restrict__ w, float eps, const void *__restrict__ gate,
+                           int gate_dtype, int gate_stride, int gate_off, int heads, int dv, int act, float mul) {
+    __shared__ float red_s[4];
+    const size_t t = blockIdx.x;
+    for (int h = 0; h < heads; ++h) {
+        const size_t base = (t * heads + h) * dv;
+        float inv = 1.f;
+        if (w) {
+            float sq = 0.f;
+            for (int j = threadIdx.x; j < dv; j += blockDim.x) {
+                const float v = rec_ld(x, x_dtype, base + j);
+                sq += v * v;
+            }
+            inv = 1.0f / sqrtf(block_sum(sq, red_s, blockDim.x / KVA_WAVE) / (float)dv + eps);
+        }
+        for (int j = threadIdx.x; j < dv; j += blockDim.x) {
+            float v = rec_ld(x, x_dtype, base + j);
+            if (w) v = v * inv * w[j];
+            const float g = rec_ld(gate, gate_dtype, t * gate_stride + gate_off + h * dv + j);
+            v *= (act == 1 ? rec_sigmoid(g) : rec_silu(g)) * mul;
+            rec_st(out, out_dtype, t * out_stride + out_off + h * dv + j, v);
+        }
+    }
+}
+
 extern "C" int kva_head_norm_gate(void *out, int out_dtype, int out_stride, int out_off, const void *x, int x_dtype,
                                   const float *w, float eps, const void *gate, int gate_dtype, int gate_stride,
                                   int gate_off, int rows, int heads, int dv, int act, float mul, hipStream_t stream) {
     KVA_REQUIRE(out && x && gate && heads > 0 && dv > 0 && rows >= 0, "head_norm_gate: missing operand or bad sizes");
     KVA_REQUIRE(act == 0 || act == 1, "head_norm_gate: activation %d is neither silu (0) nor sigmoid (1)", act);
     if (rows == 0) return KVA_OK;
-    hipLaunchKernelGGL(head_norm_gate_kernel, dim3(rows), dim3(256), 0, stream, out, out_dtype, out_stride, out_off, x,
-                       x_dtype, w, eps, gate, gate_dtype, gate_stride, gate_off, heads, dv, act, mul);
+    if (heads < 4 && dv >= 256)
+        hipLaunchKernelGGL(head_norm_gate_wide_kernel, dim3(rows), dim3(256), 0, stream, out, out_dtype, out_stride, out_off,
+                           x, x_dtype, w, eps, gate, gate_dtype, gate_stride, gate_off, heads, dv, act, mul);
+    else
+        hipLaunchKernelGGL(head_norm_gate_kernel, dim3(rows), dim3(256), 0, stream, out, out_dtype, out_stride, out_off, x,
+                           x_dtype, w, eps, gate, gate_dtype, gate_stride, gate_off, heads, dv, act, mul);
     KVA_CHECK_LAUNCH("head_norm_gate");
     return KVA_OK;
 }

@@ -69,6 +69,8 @@ _LDS_TARGET_GROUPS = 1024
 _LDS_MIN_KEYS_PER_SPLIT = 1024
 
 
+# chunked masks go to the tuned kernels where those take the head size (False: to the general rows kernel)
+CHUNKS_IN_TUNED_KERNELS = True
 _ROWS_TWO_TILES = 32 * 1024          # (token, head) rows of a step from which the general rows kernel takes two tiles an item
 
 
@@ -369,9 +371,10 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
 
     ``keep_first`` (with a window: the first so many positions stay visible behind it), ``sinks``
     (fp32 per query head: one more term exp(sink) in every denominator), a ``value_dim`` other
-    than ``head_dim`` and ``chunk`` (positions see each other only inside runs of so many positions
-    counted from 0; not together with a window) are taken by a matrix-core kernel of their own (16 rows of (token, head)
-    pairs a wavefront; bf16, head sizes with an instance) or else by the plain kernel."""
+    than ``head_dim`` are taken by a matrix-core kernel of their own (16 rows of (token, head)
+    pairs a wavefront; bf16, head sizes with an instance) or else by the plain kernel.  ``chunk``
+    (positions see each other only inside runs of so many positions counted from 0; not together with
+    a window) goes with all kernels."""
     if kv is None:
         raise K.KernelError("paged_attention: the mixer has no cache view")
     value_dim = head_dim if value_dim is None else int(value_dim)
@@ -382,7 +385,12 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
         raise K.KernelError("paged_attention: either a window or chunks")
     # the queries may be the first columns of a wider buffer: rows lie ``stride`` elements apart
     stride = qkv.stride(0)
-    if keep_first > 0 or sinks is not None or value_dim != head_dim or chunk > 0:
+    tuned = qkv.dtype == torch.bfloat16 and K.attention_mfma_supported(head_dim, kv.page_size) and stride % 8 == 0
+    if chunk > 0 and not CHUNKS_IN_TUNED_KERNELS:
+        tuned_for_chunks = False
+    else:
+        tuned_for_chunks = tuned
+    if keep_first > 0 or sinks is not None or value_dim != head_dim or (chunk > 0 and (not tuned_for_chunks or rope is not None or max_parts)):
         if rope is not None or max_parts:
             raise K.KernelError("paged_attention: kept first positions, sinks, chunks and a value size of its own "
                                 "go with neither rotation inside the kernel nor partial results")
@@ -413,11 +421,12 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
         return K.attention_mfma_rope(qkv, out, kv.k_cache, kv.v_cache, kv.block_table, meta, num_q_heads,
                                      num_kv_heads, head_dim, scale, rope[0], rope[1],
                                      kv.slot_mapping if kv.writes else None, window, splits, per, keep_cached, waves)
-    if not (qkv.dtype == torch.bfloat16 and K.attention_mfma_supported(head_dim, kv.page_size)
-            and stride % 8 == 0):
+    if not tuned:
         return K.attention_rowwise(qkv, stride, out, kv.k_cache, kv.v_cache, kv.block_table,
                                    batch.tok_seat, batch.positions, num_q_heads, num_kv_heads,
                                    head_dim, scale, window)
+    if chunk > 0:
+        window = -chunk         # the tuned kernels take both masks in one number: below zero, chunks of so many positions
     plan = _plan_for(batch, kv, num_q_heads, num_kv_heads, head_dim, max_parts)
     for launch in plan:
         if launch[0] == "wave":

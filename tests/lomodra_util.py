@@ -133,7 +133,7 @@ def bf16_rounding(t):
 
 
 def expected_rows(cfg: dict, state: Dict[str, torch.Tensor], requests: Dict[str, List[int]], routes=None,
-                  dtype: str = "float32") -> Dict[str, np.ndarray]:
+                  dtype: str = "float32", close_call: Optional[float] = None) -> Dict[str, np.ndarray]:
     """Logits of the plain forward pass per request.  With ``routes`` (what the engine's routers chose)
     the plain experts are the engine's, and every choice that differs from the plain router's own
     must be a close call of that router."""
@@ -154,7 +154,7 @@ def expected_rows(cfg: dict, state: Dict[str, torch.Tensor], requests: Dict[str,
         if forced is not None:
             for layer, (own, margin) in margins.items():
                 differs = (forced[layer].sort(-1).values != own.sort(-1).values).any(-1)
-                assert (margin[differs] <= CLOSE_CALL[dtype]).all(), \
+                assert (margin[differs] <= (CLOSE_CALL[dtype] if close_call is None else close_call)).all(), \
                     f"request {rid}, layer {layer}: the engine's router chose other experts where the choice was clear"
     return out
 

@@ -42,9 +42,9 @@ def requests_for(name, cfg):
     return {f"{name}{i}": U.prompt(cfg, n, 100 * i + n) for i, n in enumerate(REQUESTS[name])}
 
 
-def check(eng, cfg, state, reqs, steps, dtype, what):
+def check(eng, cfg, state, reqs, steps, dtype, what, close_call=None):
     rows, routes = U.run_steps(eng, steps, cfg)
-    U.assert_rows(rows, U.expected_rows(cfg, state, reqs, routes, dtype), dtype, what)
+    U.assert_rows(rows, U.expected_rows(cfg, state, reqs, routes, dtype, close_call), dtype, what)
     eng.cache.check()
     return rows
 
@@ -145,23 +145,33 @@ def _one_key_stands_out(state, layer: str, cfg_layer: dict, gain: float):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_sharp_scores_at_chunk_edges_and_far_keys(dtype, tmp_path, gpu):
+@pytest.mark.parametrize("name, gain, cuts", [("A", 4.0, (24, 23, 2, 7, 6, 8, 48, 1, 21)),
+                                              ("C", 2.0, (32, 31, 2, 16, 15, 18, 100, 1, 47, 96))])
+def test_sharp_scores_at_chunk_edges_and_far_keys(name, gain, cuts, dtype, tmp_path, gpu):
     """With sharp softmaxes every row depends on WHICH keys it sees: the positions just inside and just
     outside every chunk edge, in prompts, in portions that end and start at the edges and one token off
-    them, and decoded one by one; and - in the layer without a mask - a key hundreds of positions back."""
-    cfg = U.CFG_A
+    them, and decoded one by one; and - in the layers without a mask - a key hundreds of positions back.
+    (A: the kernels for values of another size than the keys; C: the bf16 engine's tuned kernels.)"""
+    cfg = U.CONFIGS[name][0]
 
     def edit(state):
-        for i in (0, 2, 4):
-            _one_key_stands_out(state, f"l{i}", cfg["layers"][i], 4.0)
+        for i, layer in enumerate(cfg["layers"]):
+            if layer["type"] == "attention":
+                _one_key_stands_out(state, f"l{i}", layer, gain)     # (heads of 64 and 128 are sharp at half the gain)
     folder, state = U.write_model(str(tmp_path / "sharp"), cfg, 21, edit=edit)
     reqs = {"e0": U.prompt(cfg, 75, 1), "e1": U.prompt(cfg, 340, 2)}
     eng = engine_for(folder, dtype)
-    check(eng, cfg, state, reqs, R.whole(reqs), dtype, "whole")
-    # cuts at the edges of the chunks of 24 and of 7 and one token before and behind them
-    check(eng, cfg, state, reqs, R.chunked(reqs, (24, 23, 2, 7, 6, 8, 48, 1, 21)), dtype, "cuts at chunk edges")
-    check(eng, cfg, state, {"e0": reqs["e0"]}, R.tail_decoded({"e0": reqs["e0"]}, tail=60), dtype, "decoded over chunk edges")
-    check(eng, cfg, state, {"e1": reqs["e1"]}, R.tail_decoded({"e1": reqs["e1"]}, tail=20), dtype, "decoded far from the start")
+    # (softmaxes that sharp multiply the rounding of what they read, and in bfloat16 the routers behind them
+    # see it: a gap between two logits of up to 0.6 may fall the other way there; in 32-bit none may)
+    close = None if dtype == "float32" else 0.6
+    check(eng, cfg, state, reqs, R.whole(reqs), dtype, "whole", close)
+    # cuts at the edges of the chunks and one token before and behind them
+    check(eng, cfg, state, reqs, R.chunked(reqs, cuts), dtype, "cuts at chunk edges", close)
+    check(eng, cfg, state, {"e0": reqs["e0"]}, R.tail_decoded({"e0": reqs["e0"]}, tail=60), dtype, "decoded over chunk edges", close)
+    check(eng, cfg, state, {"e1": reqs["e1"]}, R.tail_decoded({"e1": reqs["e1"]}, tail=20), dtype, "decoded far from the start", close)
+    # several requests decoded side by side, each at another place of its chunk
+    side = {f"s{i}": U.prompt(cfg, n, 30 + i) for i, n in enumerate([40, 65, 110, 129])}
+    check(eng, cfg, state, side, R.mixed(side, seed=2, max_live=4, chunk_sizes=(31, 33, 17)), dtype, "decoded side by side", close)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
