@@ -52,15 +52,21 @@ def lightning(W: Dict[str, torch.Tensor], p: str, m: dict, h, eps: float, rounde
     q = silu(rounded(h @ W[p + "q"].T)).view(T, H, d)
     k = silu(rounded(h @ W[p + "k"].T)).view(T, H, d)
     v = silu(rounded(h @ W[p + "v"].T)).view(T, H, dv)
-    decay = torch.tensor([float(a) for a in m["decay"]], dtype=F)
-    S = torch.zeros(H, d, dv, dtype=F)
-    o = torch.zeros(T, H, dv, dtype=F)
-    for t in range(T):
-        S = decay[:, None, None] * S + k[t][:, :, None] * v[t][:, None, :]
-        o[t] = torch.einsum("hdv,hd->hv", S, q[t])
+    o = fixed_decay_steps(q, k, v, torch.tensor([float(a) for a in m["decay"]], dtype=F))
     o = rms_norm(o.reshape(T, H * dv), W[p + "norm"], eps)
     o = rounded(o * torch.sigmoid(rounded(h @ W[p + "g"].T)))
     return rounded(o @ W[p + "o"].T)
+
+
+def fixed_decay_steps(q, k, v, decay):
+    """q, k [T, H, d], v [T, H, dv], decay [H]: S_t = decay_h S_(t-1) + k_t v_t^T from S = 0; returns o_t = S_t^T q_t."""
+    T, H, d = q.shape
+    S = torch.zeros(H, d, v.shape[2], dtype=F)
+    o = torch.zeros(T, H, v.shape[2], dtype=F)
+    for t in range(T):
+        S = decay[:, None, None] * S + k[t][:, :, None] * v[t][:, None, :]
+        o[t] = torch.einsum("hdv,hd->hv", S, q[t])
+    return o
 
 
 def chunk_mask(T: int, size: Optional[int]):
@@ -91,14 +97,21 @@ def attention(W, p: str, m: dict, h, eps: float, kv, rounded=_same):
     q = rounded(h @ W[p + "q"].T).view(T, H, d)
     q = rounded(rms_norm(q, W[p + "q.norm"], eps))
     k, v = kv
-    see = chunk_mask(T, (m.get("mask") or {}).get("size"))
-    out = torch.zeros(T, H, dv, dtype=F)
+    out = softmax_attention(q, k, v, m["scale"], (m.get("mask") or {}).get("size"))
+    return rounded(rounded(out.reshape(T, H * dv)) @ W[p + "o"].T)
+
+
+def softmax_attention(q, k, v, scale: float, size: Optional[int]):
+    """q [T, H, d], k [T, G, d], v [T, G, dv]: softmax((q . k) scale) over the keys ``chunk_mask`` shows, times v."""
+    T, H = q.shape[:2]
+    G = k.shape[1]
+    see = chunk_mask(T, size)
+    out = torch.zeros(T, H, v.shape[2], dtype=F)
     for hq in range(H):
         g = hq // (H // G)
-        s = (q[:, hq] @ k[:, g].T) * m["scale"]
-        s = s.masked_fill(~see, float("-inf"))
+        s = ((q[:, hq] @ k[:, g].T) * scale).masked_fill(~see, float("-inf"))
         out[:, hq] = torch.softmax(s, dim=-1) @ v[:, g]
-    return rounded(rounded(out.reshape(T, H * dv)) @ W[p + "o"].T)
+    return out
 
 
 def causal_conv(x, w):
@@ -109,6 +122,23 @@ def causal_conv(x, w):
     for j in range(taps):
         out = out + pad[j:j + T] * w[:, j]
     return out
+
+
+def delta_rule_steps(q, k, v, beta, g):
+    """q, k [T, G, d] (already unit vectors), v [T, H, dv], beta [T, H], g [T, H, d]; from S = 0, per head and
+    token in this order: S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q."""
+    T, G, d = q.shape
+    H, dv = v.shape[1], v.shape[2]
+    S = torch.zeros(H, d, dv, dtype=F)
+    o = torch.zeros(T, H, dv, dtype=F)
+    for t in range(T):
+        for hh in range(H):
+            kk, qq = k[t, hh // (H // G)], q[t, hh // (H // G)]
+            S[hh] = g[t, hh][:, None] * S[hh]
+            u = beta[t, hh] * (v[t, hh] - S[hh].T @ kk)
+            S[hh] = S[hh] + kk[:, None] * u[None, :]
+            o[t, hh] = S[hh].T @ qq
+    return o
 
 
 def channel_delta(W, p: str, m: dict, h, eps: float, rounded=_same):
@@ -123,15 +153,7 @@ def channel_delta(W, p: str, m: dict, h, eps: float, rounded=_same):
     beta = torch.sigmoid(rounded(h @ W[p + "b"].T))                                    # [T, H]
     z = rounded(h @ W[p + "a1"].T) @ W[p + "a2"].T + W[p + "dt_bias"]                   # [T, H d]
     g = torch.exp(-torch.exp(W[p + "A_log"])[None, :, None] * softplus(z).view(T, H, d))
-    S = torch.zeros(H, d, dv, dtype=F)
-    o = torch.zeros(T, H, dv, dtype=F)
-    for t in range(T):
-        for hh in range(H):
-            kk, qq = k[t, hh // (H // G)], q[t, hh // (H // G)]
-            S[hh] = g[t, hh][:, None] * S[hh]
-            u = beta[t, hh] * (v[t, hh] - S[hh].T @ kk)
-            S[hh] = S[hh] + kk[:, None] * u[None, :]
-            o[t, hh] = S[hh].T @ qq
+    o = delta_rule_steps(q, k, v, beta, g)
     o = o / rms(o, eps) * W[p + "norm"]
     gate = torch.sigmoid(rounded(rounded(h @ W[p + "g1"].T) @ W[p + "g2"].T)).view(T, H, dv)
     return rounded(rounded((o * gate).reshape(T, H * dv)) @ W[p + "o"].T)

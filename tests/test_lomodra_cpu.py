@@ -1,0 +1,191 @@
+"""Lomodra on the CPU: the configuration reader, the model as data (run order, cache and state
+slots, tensor names), and the plain implementation's mechanisms pinned against other formulations
+of the same equations."""
+import copy
+import math
+
+import pytest
+import torch
+
+import lomodra_util as U
+import plain_lomodra as plain
+from kv_cache_optimization_for_llm_amd.config.model_config import ConfigError
+from kv_cache_optimization_for_llm_amd.models.builder import Model, spec_for_config, tensor_specs_for_config
+
+F = torch.float64
+
+
+def test_a_layer_without_keys_of_its_own_reads_the_other_layers_slot():
+    cfg, spec = spec_for_config(U.CFG_A)
+    assert [c.layer for c in spec.order] == [0, 1, 2, 3, 4]
+    assert [c.cache for c in spec.order] == [0, 1, 0, 3, 0]
+    assert [c.writes_cache for c in spec.order] == [True, True, False, True, False]
+    model = Model(spec, torch.float32, "cpu")
+    groups, states = model.cache_requirements()
+    assert [sorted(slots) for _, slots in groups] == [[0]]          # one set of pages serves three layers
+    kv = groups[0][0]
+    assert kv.kind == "full" and kv.bytes_per_token(torch.bfloat16) == 2 * 2 * (32 + 16)      # keys of 32, values of 16
+    assert sorted(states) == [1, 3]
+    assert states[1].shape == (3 * 16 * 8,)                          # lightning: S of three heads
+    # delta rule: S of four heads of 16 x 24 and two earlier inputs of 2 * 2 * 16 + 4 * 24 channels
+    assert states[3].shape == (4 * 16 * 24 + 2 * 160,)
+    assert spec.residual_dtype == "float32" and model.stream_dtype == torch.float32 and spec.logit_softcap == 9.0
+
+
+def test_a_model_without_attention_has_no_pages_and_one_without_extras_runs():
+    _, spec = spec_for_config(U.CFG_D)
+    groups, states = Model(spec, torch.float32, "cpu").cache_requirements()
+    assert groups == [] and sorted(states) == [0, 1, 2]
+    _, spec = spec_for_config(U.CFG_B)
+    assert spec.logit_softcap == 0.0
+    names = tensor_specs_for_config(U.CFG_B)
+    assert "side.embed" not in names and not any(".side." in n for n in names)
+
+
+def test_tensor_names_and_shapes():
+    specs = tensor_specs_for_config(U.CFG_A)
+    assert specs["embed"].shape == (211, 96) and specs["final.norm"].shape == (96,) and "head" not in specs
+    assert specs["side.embed"].shape == (211, 5 * 12)
+    assert specs["l0.side.gate"].shape == (12, 96) and specs["l0.side.proj"].shape == (96, 12) and specs["l4.side.norm"].shape == (96,)
+    assert specs["l0.mix.q"].shape == (128, 96) and specs["l0.mix.k"].shape == (64, 96) and specs["l0.mix.v"].shape == (32, 96)
+    assert specs["l0.mix.q.norm"].shape == (32,) and specs["l0.mix.k.norm"].shape == (32,) and specs["l0.mix.o"].shape == (96, 64)
+    # layers 2 and 4 take layer 0's keys and values: queries, their norm and the output matrix only
+    assert sorted(n for n in specs if n.startswith("l2.mix.")) == ["l2.mix.o", "l2.mix.q", "l2.mix.q.norm"]
+    assert specs["l1.mix.q"].shape == (48, 96) and specs["l1.mix.v"].shape == (24, 96) and specs["l1.mix.norm"].shape == (24,)
+    assert specs["l1.mix.g"].shape == (24, 96) and "l1.mix.decay" not in specs      # the decays are constants of the configuration
+    assert not any(n.startswith("l1.mlp") for n in specs) and "l1.norm1" in specs
+    assert specs["l3.mix.q"].shape == (32, 96) and specs["l3.mix.v"].shape == (96, 96) and specs["l3.mix.v.conv"].shape == (96, 3)
+    assert specs["l3.mix.b"].shape == (4, 96) and specs["l3.mix.a1"].shape == (6, 96) and specs["l3.mix.a2"].shape == (64, 6)
+    assert specs["l3.mix.dt_bias"].shape == (64,) and specs["l3.mix.A_log"].shape == (4,) and specs["l3.mix.norm"].shape == (24,)
+    assert specs["l3.mix.g1"].shape == (5, 96) and specs["l3.mix.g2"].shape == (96, 5)
+    assert specs["l0.mlp.router"].shape == (5, 96) and specs["l0.mlp.router.b"].shape == (5,)
+    assert specs["l0.mlp.e4.gate"].shape == (48, 96) and specs["l0.mlp.e4.down"].shape == (96, 48) and "l0.mlp.e5.up" not in specs
+    assert specs["l0.mlp.shared.up"].shape == (40, 96) and "l3.mlp.shared.up" not in specs
+    free = copy.deepcopy(U.CFG_A)
+    del free["layers"][3]["mixer"]["decay_rank"], free["layers"][3]["mixer"]["gate_rank"]
+    specs = tensor_specs_for_config(free)                            # the stored tensors give the inner sizes
+    assert specs["l3.mix.a1"].shape == (None, 96) and specs["l3.mix.g2"].shape == (96, None)
+
+
+@pytest.mark.parametrize("edit, message", [
+    (lambda c: c["layers"][0].update(type="conv"), "type"),
+    (lambda c: c["layers"][0]["mixer"].update(kv_heads=3), "multiple"),
+    (lambda c: c["layers"][0]["mixer"].pop("scale"), "scale"),
+    (lambda c: c["layers"][0]["mixer"]["mask"].update(size=0), "mask.size"),
+    (lambda c: c["layers"][0]["mixer"].update(dim=30), "multiple of 4"),
+    (lambda c: c["layers"][1]["mixer"].update(decay=[0.5, 0.9]), "decay"),
+    (lambda c: c["layers"][2]["mixer"].update(kv_from=2), "earlier"),
+    (lambda c: c["layers"][2]["mixer"].update(kv_from=1), "no keys and values"),
+    (lambda c: c["layers"][4]["mixer"].update(kv_from=2), "no keys and values"),
+    (lambda c: c["layers"][2]["mixer"].update(vdim=8), "sizes differ"),
+    (lambda c: c["layers"][3]["mixer"].update(conv=0), "conv"),
+    (lambda c: c["layers"][0]["mlp"]["router"].update(top=6), "top"),
+    (lambda c: c["layers"][0]["mlp"].update(kind="dense"), "kind"),
+    (lambda c: c["token_side"].update(dim=0), "token_side"),
+    (lambda c: c.update(logit_softcap=-1.0), "logit_softcap"),
+    (lambda c: c.pop("norm"), "eps"),
+    (lambda c: c.update(layers=[]), "layers"),
+])
+def test_a_configuration_that_cannot_run_is_refused(edit, message):
+    cfg = copy.deepcopy(U.CFG_A)
+    edit(cfg)
+    with pytest.raises(ConfigError, match=message):
+        spec_for_config(cfg)
+
+
+def test_fixed_decay_as_a_sum_over_earlier_tokens():
+    g = torch.Generator().manual_seed(1)
+    T, H, d, dv = 9, 3, 5, 4
+    q, k, v = (torch.randn(T, H, n, generator=g, dtype=F) for n in (d, d, dv))
+    decay = torch.tensor([1.0, 0.5, 0.9], dtype=F)
+    out = plain.fixed_decay_steps(q, k, v, decay)
+    for t in range(T):
+        want = torch.zeros(H, dv, dtype=F)
+        for j in range(t + 1):
+            want += (decay ** (t - j) * (q[t] * k[j]).sum(-1))[:, None] * v[j]
+        torch.testing.assert_close(out[t], want)
+
+
+def test_delta_rule_with_channel_decays_as_matrices():
+    """S <- (I - beta k k^T) diag(g) S + beta k v^T; with beta = 1, no decay and orthonormal keys the
+    state returns every stored value."""
+    g = torch.Generator().manual_seed(2)
+    d, dv, T = 6, 4, 6
+    k = torch.linalg.qr(torch.randn(d, d, generator=g, dtype=F)).Q[:, None, :]
+    v = torch.randn(T, 1, dv, generator=g, dtype=F)
+    out = plain.delta_rule_steps(k, k, v, torch.ones(T, 1, dtype=F), torch.ones(T, 1, d, dtype=F))
+    torch.testing.assert_close(out, v)
+    H = 2                                                       # two heads on one q/k head
+    q, kk = torch.randn(T, 1, d, generator=g, dtype=F), torch.randn(T, 1, d, generator=g, dtype=F)
+    v = torch.randn(T, H, dv, generator=g, dtype=F)
+    beta, dec = torch.rand(T, H, generator=g, dtype=F), torch.rand(T, H, d, generator=g, dtype=F)
+    out = plain.delta_rule_steps(q, kk, v, beta, dec)
+    for h in range(H):
+        S = torch.zeros(d, dv, dtype=F)
+        for t in range(T):
+            S = (torch.eye(d, dtype=F) - beta[t, h] * torch.outer(kk[t, 0], kk[t, 0])) @ (dec[t, h][:, None] * S) \
+                + beta[t, h] * torch.outer(kk[t, 0], v[t, h])
+            torch.testing.assert_close(out[t, h], S.T @ q[t, 0])
+
+
+def test_chunks_are_attention_over_each_chunk_alone():
+    g = torch.Generator().manual_seed(3)
+    T, H, G, d, dv, size = 23, 4, 2, 6, 5, 7
+    q, k, v = torch.randn(T, H, d, generator=g, dtype=F), torch.randn(T, G, d, generator=g, dtype=F), torch.randn(T, G, dv, generator=g, dtype=F)
+    whole = plain.softmax_attention(q, k, v, 0.4, size)
+    for lo in range(0, T, size):
+        hi = min(T, lo + size)
+        torch.testing.assert_close(whole[lo:hi], plain.softmax_attention(q[lo:hi], k[lo:hi], v[lo:hi], 0.4, None))
+    see = plain.chunk_mask(T, size)
+    assert see[13, 7] and not see[13, 6] and see[14, 14] and not see[14, 13] and not see[6, 7] and see[6, 0]
+    assert torch.equal(plain.chunk_mask(T, None), torch.ones(T, T).tril().bool())
+    assert torch.equal(plain.chunk_mask(T, 1), torch.eye(T).bool())
+    assert torch.equal(plain.chunk_mask(T, T + 5), plain.chunk_mask(T, None))
+
+
+def test_causal_convolution_against_conv1d():
+    g = torch.Generator().manual_seed(4)
+    x, w = torch.randn(11, 6, generator=g, dtype=F), torch.randn(6, 4, generator=g, dtype=F)
+    want = torch.nn.functional.conv1d(torch.nn.functional.pad(x.T[None], (3, 0)), w[:, None, :], groups=6)[0].T
+    torch.testing.assert_close(plain.causal_conv(x, w), want)
+    torch.testing.assert_close(plain.causal_conv(x, w[:, -1:]), x * w[:, -1])     # one tap: the current token's alone
+
+
+def test_weights_over_the_chosen_logits_and_the_expert_every_token_uses():
+    g = torch.Generator().manual_seed(5)
+    Wd, ff, E = 8, 4, 5
+    W = {"m.router": torch.randn(E, Wd, generator=g, dtype=F), "m.router.b": torch.tensor([0.0, 0.0, 50.0, 0.0, 49.0], dtype=F)}
+    for e in list(range(E)) + ["s"]:
+        p = "m.shared." if e == "s" else f"m.e{e}."
+        W[p + "gate"], W[p + "up"], W[p + "down"] = (torch.randn(s, generator=g, dtype=F) for s in ((ff, Wd), (ff, Wd), (Wd, ff)))
+    h = torch.randn(6, Wd, generator=g, dtype=F)
+    mlp = {"router": {"experts": E, "top": 2}, "shared": {"ff": ff}}
+    out = plain.mixture(W, "m.", mlp, h)
+    z = plain.router_logits(W, "m.", h)
+    a = torch.softmax(z, -1)                                    # the same weights: a softmax over all, renormalised over the chosen
+    w2, w4 = a[:, 2] / (a[:, 2] + a[:, 4]), a[:, 4] / (a[:, 2] + a[:, 4])
+    one = lambda p: (plain.silu(h @ W[p + "gate"].T) * (h @ W[p + "up"].T)) @ W[p + "down"].T
+    torch.testing.assert_close(out, w2[:, None] * one("m.e2.") + w4[:, None] * one("m.e4.") + one("m.shared."))
+    W["m.router.b"] = torch.tensor([0.0, 0.0, 100.0, 0.0, 0.0], dtype=F)      # one choice: its weight is 1
+    torch.testing.assert_close(plain.mixture(W, "m.", {"router": {"experts": E, "top": 1}, "shared": None}, h), one("m.e2."))
+    assert plain.gelu_tanh(torch.tensor(1.0, dtype=F)).item() == pytest.approx(
+        0.5 * (1 + math.tanh(math.sqrt(2 / math.pi) * 1.044715)))
+    assert plain.softplus(torch.tensor([-800.0, 0.0, 800.0], dtype=F)).tolist() == pytest.approx([0.0, math.log(2.0), 800.0])
+
+
+def test_the_whole_model_in_pieces_equals_the_whole_model(tmp_path):
+    """Logits at a position do not depend on what follows (every mechanism is causal), and the layers'
+    outputs are what the logits are made of."""
+    for name in ("A", "B"):
+        cfg = U.CONFIGS[name][0]
+        folder, state = U.write_model(str(tmp_path / name), cfg, 3)
+        W = plain.to_f64(state)
+        toks = U.prompt(cfg, 30, 1)
+        layers = []
+        full = plain.forward(cfg, W, toks, layer_outputs=layers)
+        torch.testing.assert_close(plain.forward(cfg, W, toks[:9]), full[:9])
+        assert len(layers) == len(cfg["layers"])
+        logits = plain.rms_norm(layers[-1], W["final.norm"], cfg["norm"]["eps"]) @ W["embed"].T
+        cap = cfg.get("logit_softcap")
+        torch.testing.assert_close(full, cap * torch.tanh(logits / cap) if cap else logits)
+        assert not cap or full.abs().max() < cap

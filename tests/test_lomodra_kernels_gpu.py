@@ -1,0 +1,386 @@
+"""The kernels behind the Lomodra parts, each alone against a plain function of ``plain_lomodra``:
+the router whose weights are a softmax over the chosen logits, gated experts beside an expert every
+token uses, the recurrence with one fixed decay a head (cut into steps, seats used again, a far
+token), the delta rule with a decay per key channel and the epilogue that makes those decays, the
+norm on a branch's way into the stream, the gate times a token's table columns, the per-head RMS
+norm of queries and keys with its cache write, one norm over all heads of a row, and softmax
+attention confined to chunks of positions (a key that stands out just inside and just outside)."""
+import numpy as np
+import pytest
+import torch
+
+import plain_lomodra as plain
+from kv_cache_optimization_for_llm_amd.ops import kernels as K
+from test_gadopel_kernels_gpu import cache_for, standout
+from test_radilix_kernels_gpu import cuts, dev, ints, run_in_steps  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+F = torch.float64
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def rnd(shape, seed, std=1.0):
+    return torch.randn(shape, generator=torch.Generator().manual_seed(seed)) * std
+
+
+# ---- router -----------------------------------------------------------------------------------
+@pytest.mark.parametrize("outputs, top", [(1, 1), (2, 1), (5, 5), (7, 2), (64, 8), (65, 3), (300, 6)])
+def test_router_weights_are_a_softmax_over_the_chosen_logits(outputs, top, gpu):
+    logits = rnd((83, outputs), outputs * 7 + top, 2.5)
+    idx = torch.empty((83, top), dtype=torch.int32, device="cuda")
+    wgt = torch.empty((83, top), dtype=torch.float32, device="cuda")
+    K.moe_route(dev(logits), None, top, idx, wgt, over_chosen=True)
+    z = logits.to(F)
+    ordered = torch.sort(z, dim=-1, descending=True).values
+    clear = (ordered[:, top - 1] - ordered[:, top] > 1e-6) if top < outputs else torch.ones(83, dtype=torch.bool)
+    own = torch.topk(z, top, dim=-1).indices
+    got = idx.cpu().long()
+    assert torch.equal(got[clear].sort(-1).values, own[clear].sort(-1).values)
+    want = torch.softmax(torch.gather(z, 1, got), dim=-1)
+    torch.testing.assert_close(wgt.cpu().to(F), want, rtol=2e-5, atol=1e-7)
+    torch.testing.assert_close(wgt.sum(-1).cpu(), torch.ones(83), rtol=1e-5, atol=1e-6)
+
+
+# ---- gated experts beside an expert every token uses ---------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width, ff, experts, top, shared, tokens",
+                         [(64, 32, 4, 2, 48, 1), (64, 96, 7, 3, 0, 50), (72, 40, 3, 3, 8, 33), (96, 48, 1, 1, 96, 17),
+                          (128, 160, 16, 4, 64, 300), (40, 24, 2, 1, 0, 9), (64, 520, 4, 2, 32, 1100)])
+def test_gated_experts_against_the_plain_mixture(width, ff, experts, top, shared, tokens, dtype, gpu):
+    from kv_cache_optimization_for_llm_amd.parts.base import MixerContext
+    from kv_cache_optimization_for_llm_amd.parts.moe import RoutedExperts
+    g = torch.Generator().manual_seed(width + ff + experts + tokens)
+    part = RoutedExperts("m.", hidden_size=width, intermediate_size=ff, experts=experts, top=top, activation="silu",
+                         correction=False, gated=True, router_bias=True, softmax_over="chosen", shared_intermediate=shared)
+    W = {}
+    for name, spec in part.tensor_specs().items():
+        std = 0.5 if name.endswith("router.b") else (1.0 / spec.shape[-1] ** 0.5)
+        W[name] = (torch.randn(spec.shape, generator=g) * std).to(torch.bfloat16)
+    assert ("m.shared.gate" in W) == (shared > 0) and f"m.e{experts - 1}.gate" in W and "m.router.b" in W
+    part.load({k: dev(v, dtype) for k, v in W.items()})
+    x = torch.randn(tokens, width, generator=g).to(torch.bfloat16)
+    seen = []
+    RoutedExperts.on_route = lambda p, idx: seen.append(idx.cpu().long())
+    try:
+        got = part.forward(dev(x, dtype), MixerContext(batch=None))
+    finally:
+        RoutedExperts.on_route = None
+    mlp = {"router": {"experts": experts, "top": top}, "shared": {"ff": shared} if shared else None}
+    margins = []
+    want = plain.mixture(plain.to_f64(W), "m.", mlp, x.to(F), choices=seen[0], margin_out=margins)
+    own, margin = margins[0]
+    differs = (seen[0].sort(-1).values != own.sort(-1).values).any(-1)
+    assert (margin[differs] < (1e-5 if dtype == torch.float32 else 2e-2)).all()
+    tol = dict(rtol=2e-5, atol=2e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(got.cpu().to(F), want, **tol)
+
+
+# ---- one fixed decay a head ------------------------------------------------------------------------
+@pytest.mark.parametrize("heads, dim, vdim", [(4, 48, 32), (1, 16, 16), (3, 20, 9), (2, 128, 40), (5, 8, 64), (2, 144, 18), (1, 100, 5)])
+@pytest.mark.parametrize("portions", [(1000,), (1,), (3, 1, 16, 2, 50), (31, 33, 32, 1)])
+def test_fixed_decay_recurrence_over_steps(heads, dim, vdim, portions, gpu):
+    g = torch.Generator().manual_seed(heads * dim + vdim + 2)
+    lengths = {1: 97, 0: 5, 2: 32}
+    q_off, k_off, v_off = 3, 3 + heads * dim, 3 + 2 * heads * dim
+    ycols = v_off + heads * vdim + 2
+    y = {s: torch.randn(n, ycols, generator=g) for s, n in lengths.items()}
+    decay = torch.tensor([1.0, 0.5, 0.97, 0.999, 0.8][:heads])
+    state = torch.zeros((3, 4 + heads * dim * vdim), dtype=torch.float32, device="cuda")
+
+    def launch(seats, lens, starts):
+        ys = torch.cat([y[s][a:a + n] for s, n, a in zip(seats, lens, starts)])
+        out = torch.empty((ys.shape[0], heads * vdim), dtype=torch.float32, device="cuda")
+        return K.gated_linear_attention(dev(ys), q_off, k_off, v_off, None, 1.0, out, state, 4, ints(np.cumsum([0] + lens)),
+                                        ints(seats), heads, dim, vdim, head_decay=dev(decay), activation="silu")
+    got = run_in_steps(lengths, portions, launch)
+    for s, n in lengths.items():
+        r = plain.silu(y[s].to(F))
+        want = plain.fixed_decay_steps(r[:, q_off:q_off + heads * dim].view(n, heads, dim),
+                                       r[:, k_off:k_off + heads * dim].view(n, heads, dim),
+                                       r[:, v_off:v_off + heads * vdim].view(n, heads, vdim), decay.to(F))
+        torch.testing.assert_close(got[s].to(F), want.reshape(n, -1), rtol=2e-4, atol=2e-4)
+    assert (state[:, :4] == 0).all()
+
+
+def test_fixed_decay_without_activation_and_with_a_query_scale(gpu):
+    heads, dim, vdim, n = 2, 32, 16, 40
+    y = rnd((n, 2 * heads * dim + heads * vdim), 5)
+    decay = torch.tensor([0.9, 0.6])
+    state = torch.zeros((1, heads * dim * vdim), dtype=torch.float32, device="cuda")
+    out = torch.empty((n, heads * vdim), dtype=torch.float32, device="cuda")
+    K.gated_linear_attention(dev(y), 0, heads * dim, 2 * heads * dim, None, 0.25, out, state, 0, ints([0, n]), ints([0]),
+                             heads, dim, vdim, head_decay=dev(decay), activation=None)
+    r = y.to(F)
+    want = plain.fixed_decay_steps(r[:, :heads * dim].view(n, heads, dim) * 0.25, r[:, heads * dim:2 * heads * dim].view(n, heads, dim),
+                                   r[:, 2 * heads * dim:].view(n, heads, vdim), decay.to(F))
+    torch.testing.assert_close(out.cpu().to(F), want.reshape(n, -1), rtol=2e-4, atol=2e-4)
+
+
+# ---- a decay per head and key channel -------------------------------------------------------------
+@pytest.mark.parametrize("tokens, heads, dim, rank", [(1, 2, 16, 4), (9, 3, 20, 7), (33, 4, 64, 16), (5, 1, 160, 3), (70, 6, 8, 1)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_decays_from_a_low_rank_product_with_a_rate_a_head(tokens, heads, dim, rank, dtype, gpu):
+    g = torch.Generator().manual_seed(heads * dim + rank)
+    wide = (torch.randn(tokens, rank + 9, generator=g) * 2).to(dtype)
+    a2 = torch.randn(heads * dim, rank, generator=g).to(dtype)
+    bias, a_log = torch.randn(heads * dim, generator=g), torch.randn(heads, generator=g) * 0.7 - 1.0
+    out = torch.empty((tokens, heads * dim), dtype=torch.float32, device="cuda")
+    K.small_product_f32(dev(wide, dtype)[:, 4:4 + rank], dev(a2, dtype), out, bias=dev(bias), rate_log=dev(a_log))
+    z = wide[:, 4:4 + rank].to(F) @ a2.to(F).T + bias.to(F)
+    want = torch.exp(-torch.exp(a_log.to(F))[None, :, None] * plain.softplus(z).view(tokens, heads, dim)).reshape(tokens, -1)
+    torch.testing.assert_close(out.cpu().to(F), want, rtol=2e-5, atol=1e-6)
+    assert (out > 0).all() and (out <= 1).all()
+
+
+@pytest.mark.parametrize("heads, kv_heads, dim, vdim", [(2, 1, 32, 32), (4, 2, 16, 24), (3, 3, 20, 7), (2, 2, 128, 48), (6, 2, 8, 70), (2, 1, 160, 20), (1, 1, 64, 3)])
+@pytest.mark.parametrize("portions", [(1000,), (1,), (2, 1, 17, 5, 64), (32, 31, 1, 33)])
+def test_delta_rule_with_channel_decays_over_steps(heads, kv_heads, dim, vdim, portions, gpu):
+    g = torch.Generator().manual_seed(heads * dim + vdim + 7)
+    lengths = {2: 131, 0: 9, 1: 64}
+    C = 2 * kv_heads * dim + heads * vdim
+    ycols, boff = heads + 3, 2
+    qkv = {s: torch.randn(n, C, generator=g) for s, n in lengths.items()}
+    y = {s: torch.randn(n, ycols, generator=g) * 2 for s, n in lengths.items()}
+    # decays spread over (0, 1]: some channels forget at once, some keep nearly all
+    dec = {s: torch.rand(n, heads * dim, generator=g) ** 0.3 for s, n in lengths.items()}
+    state = torch.zeros((3, 4 + heads * dim * vdim), dtype=torch.float32, device="cuda")
+
+    def launch(seats, lens, starts):
+        take = lambda src: torch.cat([src[s][a:a + n] for s, n, a in zip(seats, lens, starts)])
+        rows = take(qkv)
+        out = torch.empty((rows.shape[0], heads * vdim), dtype=torch.float32, device="cuda")
+        return K.gated_delta_rule(dev(rows), dev(take(y)), boff, 0, None, None, out, state, 4, ints(np.cumsum([0] + lens)),
+                                  ints(seats), heads, kv_heads, dim, vdim, 1e-6, channel_decay=dev(take(dec)))
+    got = run_in_steps(lengths, portions, launch)
+    for s, n in lengths.items():
+        r = qkv[s].to(F)
+        unit = lambda x: x / torch.sqrt((x * x).sum(-1, keepdim=True) + 1e-6)
+        q = unit(r[:, :kv_heads * dim].view(n, kv_heads, dim)) * dim ** -0.5
+        k = unit(r[:, kv_heads * dim:2 * kv_heads * dim].view(n, kv_heads, dim))
+        v = r[:, 2 * kv_heads * dim:].view(n, heads, vdim)
+        beta = torch.sigmoid(y[s][:, boff:boff + heads].to(F))
+        want = plain.delta_rule_steps(q, k, v, beta, dec[s].to(F).view(n, heads, dim))
+        torch.testing.assert_close(got[s].to(F), want.reshape(n, -1), rtol=2e-4, atol=2e-5)
+    assert (state[:, :4] == 0).all()
+
+
+def test_a_channel_that_forgets_and_one_that_keeps(gpu):
+    """Two key channels hold one value each; the first channel's decay is 0 from the second token on and the
+    other's is 1: hundreds of tokens later a query along the second channel returns its value whole, a
+    query along the first returns nothing.  A decay per HEAD could do neither."""
+    dim, vdim, n = 16, 8, 300
+    q, k, v = torch.zeros(n, dim), torch.zeros(n, dim), torch.zeros(n, vdim)
+    k[0, 0], k[1, 1] = 1.0, 1.0
+    v[0], v[1] = torch.arange(vdim) + 10.0, torch.arange(vdim) - 20.0
+    k[2:, 5] = 1.0                                            # later keys write elsewhere (values of zero)
+    q[-2, 0], q[-1, 1] = 1.0, 1.0
+    dec = torch.ones(n, dim)
+    dec[1:, 0] = 0.0
+    y = torch.full((n, 1), 30.0)                              # beta = 1
+    state = torch.zeros((1, dim * vdim), dtype=torch.float32, device="cuda")
+    out = torch.empty((n, vdim), dtype=torch.float32, device="cuda")
+    for lo in range(0, n, 47):
+        hi = min(n, lo + 47)
+        K.gated_delta_rule(dev(torch.cat([q, k, v], 1)[lo:hi]), dev(y[lo:hi]), 0, 0, None, None, out[lo:hi], state, 0,
+                           ints([0, hi - lo]), ints([0]), 1, 1, dim, vdim, 1e-6, channel_decay=dev(dec[lo:hi]))
+    torch.testing.assert_close(out[-1].cpu(), v[1] * dim ** -0.5, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(out[-2].cpu(), torch.zeros(vdim), rtol=0, atol=1e-5)
+
+
+def test_a_far_token_under_a_decay_of_one_and_a_seat_taken_again(gpu):
+    dim, vdim, n = 16, 16, 600
+    y = torch.zeros(n, 2 * dim + vdim)
+    big = 30.0                                                # silu(30) = 30
+    y[0, dim] = big                                           # key 0 along channel 0
+    y[0, 2 * dim:] = torch.arange(vdim) + 1.0
+    for t in range(1, n):
+        y[t, dim + 1 + t % (dim - 1)] = 1.0                   # other keys avoid channel 0
+        y[t, 2 * dim:] = 3.0
+    y[-1, 0] = big
+    v0 = plain.silu(y[0, 2 * dim:].to(F))
+    state = torch.zeros((2, dim * vdim), dtype=torch.float32, device="cuda")
+    out = torch.empty((n, vdim), dtype=torch.float32, device="cuda")
+    for decay, keeps in ((1.0, 1.0), (0.99, 0.99 ** (n - 1))):
+        for _ in range(2):                                    # the second time on the seat zeroed as a new request finds it
+            state[1].zero_()
+            for lo in range(0, n, 64):
+                hi = min(n, lo + 64)
+                K.gated_linear_attention(dev(y[lo:hi]), 0, dim, 2 * dim, None, 1.0, out[lo:hi], state, 0, ints([0, hi - lo]),
+                                         ints([1]), 1, dim, vdim, head_decay=dev(torch.tensor([decay])), activation="silu")
+            torch.testing.assert_close(out[-1].cpu().to(F), v0 * big * big * keeps, rtol=3e-4, atol=1e-4)
+    assert (state[0] == 0).all()
+
+
+# ---- a branch's output normed on its way into the stream -----------------------------------------
+@pytest.mark.parametrize("width", [8, 72, 96, 256, 2048, 4104])
+@pytest.mark.parametrize("stream, branch, copy", [("float32", "float32", None), ("float32", "bfloat16", "bfloat16"),
+                                                 ("float32", "bfloat16", None), ("bfloat16", "bfloat16", "bfloat16"),
+                                                 ("float32", "float32", "float32")])
+def test_norm_into_stream(width, stream, branch, copy, gpu):
+    T, eps = 19, 0.01
+    x = rnd((T, width), width, 3.0).to(DT[stream])
+    y = rnd((T, width), width + 1, 0.5).to(DT[branch])
+    y[3] = 0.0                                               # a row of zeros stays zero: eps stands inside the root
+    w = (rnd((width,), width + 2, 0.3) + 1.0).to(DT[branch])
+    xs = dev(x, DT[stream])
+    cp = None if copy is None else torch.full((T, width), 7.0, dtype=DT[copy], device="cuda")
+    K.norm_into_stream(xs, dev(y, DT[branch]), dev(w, DT[branch]), eps, cp)
+    want = x.to(F) + plain.rms_norm(y.to(F), w.to(F), eps)
+    tol = dict(rtol=1e-5, atol=1e-5) if stream == "float32" else dict(rtol=1e-2, atol=2e-2)
+    torch.testing.assert_close(xs.cpu().to(F), want, **tol)
+    torch.testing.assert_close(xs[3].cpu(), x[3], rtol=0, atol=0)
+    if cp is not None:
+        torch.testing.assert_close(cp.cpu().to(F), xs.cpu().to(F), **(dict(rtol=0, atol=0) if copy == stream else dict(rtol=1e-2, atol=2e-2)))
+
+
+# ---- a gate times the token's columns of a table --------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dim, layers, layer", [(1, 3, 2), (12, 5, 0), (32, 7, 3), (100, 2, 1), (256, 1, 0)])
+def test_table_gate_takes_the_layers_columns_of_the_tokens_row(dim, layers, layer, dtype, gpu):
+    T, vocab = 23, 61
+    z = rnd((T, dim), dim, 2.0).to(DT[dtype])
+    table = rnd((vocab, layers * dim), dim + 1).to(DT[dtype])
+    ids = torch.randint(0, vocab, (T,), generator=torch.Generator().manual_seed(dim))
+    ids[0], ids[1] = 0, vocab - 1
+    feedback = torch.tensor([5, vocab - 1, 17], dtype=torch.int32)
+    sent = ids.clone()
+    sent[4], sent[9] = -1 - 2, -1 - 0                          # tokens that are still on the device
+    ids[4], ids[9] = 17, 5
+    out = torch.empty((T, dim), dtype=DT[dtype], device="cuda")
+    K.table_gate(dev(z, DT[dtype]), dev(table, DT[dtype]), dev(sent, torch.int32), layer * dim, out, "gelu_tanh", dev(feedback, torch.int32))
+    want = plain.gelu_tanh(z.to(F)) * table.to(F)[ids][:, layer * dim:(layer + 1) * dim]
+    tol = dict(rtol=1e-5, atol=1e-6) if dtype == "float32" else dict(rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(out.cpu().to(F), want, **tol)
+
+
+# ---- queries and keys under an RMS norm per head, keys cached normed ------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("heads, kv_heads, dim, vdim", [(4, 2, 32, 16), (3, 3, 20, 20), (2, 1, 64, 64), (8, 2, 128, 32), (2, 0, 24, 8)])
+def test_head_norms_of_queries_and_keys_and_the_cache_write(heads, kv_heads, dim, vdim, dtype, gpu):
+    T, page, eps = 29, 8, 0.03
+    table, slots, pages = cache_for(T, page, 5)
+    width = heads * dim + kv_heads * (dim + vdim)
+    y = rnd((T, width + 6), dim + heads, 2.0).to(DT[dtype])
+    wq, wk = rnd((dim,), 1, 0.3) + 1.0, rnd((dim,), 2, 0.3) + 1.0
+    k_cache = torch.zeros((pages, *K.k_page_shape(max(kv_heads, 1), dim)[:2], page, K.k_chunk(dim)), dtype=DT[dtype], device="cuda")
+    v_cache = torch.zeros((pages, max(kv_heads, 1), vdim, page), dtype=DT[dtype], device="cuda")
+    buf = dev(y, DT[dtype])
+    own = kv_heads > 0
+    K.qk_encode_cache(buf[:, :width], dev(torch.arange(T), torch.int32), heads, kv_heads, dim, vdim, None, None, False, eps,
+                      k_cache if own else None, v_cache if own else None, dev(slots, torch.int32) if own else None,
+                      q_weight=dev(wq), k_weight=dev(wk) if own else None)
+    src = y.to(F)
+    q = plain.rms_norm(src[:, :heads * dim].view(T, heads, dim), wq.to(F), eps)
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == "float32" else dict(rtol=1e-2, atol=2e-2)
+    torch.testing.assert_close(buf[:, :heads * dim].cpu().to(F), q.reshape(T, -1), **tol)
+    torch.testing.assert_close(buf[:, width:].cpu(), y[:, width:], rtol=0, atol=0)
+    if not own:
+        assert (k_cache == 0).all() and (v_cache == 0).all()
+        return
+    k = plain.rms_norm(src[:, heads * dim:(heads + kv_heads) * dim].view(T, kv_heads, dim), wk.to(F), eps)
+    v = src[:, (heads + kv_heads) * dim:width].view(T, kv_heads, vdim)
+    keys = K.pages_to_keys(k_cache).reshape(pages, kv_heads, page, dim).cpu().to(F)
+    sl = slots.long()
+    torch.testing.assert_close(keys[sl // page, :, sl % page], k, **tol)
+    torch.testing.assert_close(v_cache.cpu().to(F)[sl // page, :, :, sl % page], v, rtol=0, atol=0)
+
+
+# ---- one norm over all heads of a row ---------------------------------------------------------------
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width", [5, 24, 200, 512, 2048, 4100])
+def test_one_norm_over_the_whole_row_with_a_gate(width, out_dtype, gpu):
+    T, eps = 11, 0.02
+    x = rnd((T, width), width, 3.0)
+    gate = rnd((T, width + 9), width + 1).to(out_dtype)
+    w = rnd((width,), width + 2, 0.3) + 1.0
+    out = torch.full((T, width + 5), 7.0, dtype=out_dtype, device="cuda")
+    K.head_norm_gate(dev(x), dev(w), eps, dev(gate, out_dtype), 4, out, 2, 1, width, "sigmoid", 1.0)
+    want = plain.rms_norm(x.to(F), w.to(F), eps) * torch.sigmoid(gate[:, 4:4 + width].to(F))
+    tol = dict(rtol=1e-5, atol=1e-5) if out_dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(out[:, 2:2 + width].cpu().to(F), want, **tol)
+    assert (out[:, :2] == 7).all() and (out[:, 2 + width:] == 7).all()
+
+
+# ---- softmax attention inside chunks of positions ---------------------------------------------------
+CHUNK_CASES = [  # (length, chunk, query position, key that stands out)
+    (300, 0, 299, 0), (300, 0, 299, 157),                         # no mask: far keys
+    (300, 44, 299, 264), (300, 44, 299, 263),                    # the first key of the query's chunk / the last of the one before
+    (300, 44, 264, 264), (300, 44, 264, 263), (300, 44, 263, 220), (300, 44, 263, 219),
+    (130, 16, 129, 128), (130, 16, 129, 127), (130, 16, 127, 112), (130, 16, 127, 111),     # chunks that are pages
+    (130, 24, 47, 24), (130, 24, 47, 23), (130, 24, 48, 47), (130, 24, 48, 48),             # chunk edges inside pages
+    (70, 1, 69, 69), (70, 1, 69, 68), (70, 64, 69, 64), (70, 64, 69, 63), (70, 64, 63, 0),
+    (5, 3, 4, 3), (5, 3, 4, 2), (5, 100, 4, 0), (1, 4, 0, 0),
+]
+
+
+def chunk_reference(q, k, v, scale, chunk):
+    return plain.softmax_attention(q.to(F), k.to(F), v.to(F), scale, chunk or None)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("length, chunk, qpos, kpos", CHUNK_CASES)
+def test_plain_attention_kernel_sees_exactly_its_chunk(length, chunk, qpos, kpos, dtype, gpu):
+    heads, kv_heads, dim, vdim, page, scale = 4, 2, 24, 40, 16, 0.3
+    q, k, v = rnd((length, heads, dim), 1), rnd((length, kv_heads, dim), 2), rnd((length, kv_heads, vdim), 3)
+    standout(q, k, qpos, kpos, head=2, kv_head=1)
+    v[kpos, 1] = 5.0
+    q, k, v = (t.to(DT[dtype]) for t in (q, k, v))
+    table, slots, pages = cache_for(length, page, 11)
+    k_cache = torch.zeros((pages, *K.k_page_shape(kv_heads, dim)[:2], page, K.k_chunk(dim)), dtype=DT[dtype], device="cuda")
+    v_cache = torch.full((pages, kv_heads, vdim, page), float("nan"), dtype=DT[dtype], device="cuda")
+    sl = slots.long()
+    kp = K.pages_to_keys(k_cache).reshape(pages, kv_heads, page, dim)
+    kp[sl // page, :, sl % page] = k.to("cuda")
+    k_cache.copy_(K.keys_to_pages(kp))
+    v_cache[sl // page, :, :, sl % page] = v.to("cuda")
+    rows = sorted({qpos, 0, length - 1, length // 2, max(0, qpos - 1)})
+    out = torch.empty((len(rows), heads * vdim), dtype=DT[dtype], device="cuda")
+    K.attention_rowwise(q[rows].reshape(len(rows), -1).contiguous().to("cuda"), heads * dim, out, k_cache, v_cache,
+                        table.to("cuda"), torch.ones(len(rows), dtype=torch.int32, device="cuda"),
+                        torch.tensor(rows, dtype=torch.int32, device="cuda"), heads, kv_heads, dim, scale, 0, 0, None, vdim, chunk)
+    want = chunk_reference(q, k, v, scale, chunk)[rows].reshape(len(rows), -1)
+    assert torch.isfinite(out).all()
+    tol = 1e-4 if dtype == "float32" else 6e-2
+    torch.testing.assert_close(out.cpu().to(F), want, rtol=tol, atol=tol)
+    seen = bool(plain.chunk_mask(length, chunk or None)[qpos, kpos])
+    got = out.view(len(rows), heads, vdim)[rows.index(qpos), 2].float().mean().item()
+    assert (got > 2.5) == seen, f"the key that stands out is {'visible' if seen else 'hidden'}, the output says {got:.2f}"
+
+
+@pytest.mark.parametrize("row_tiles", [1, 2])
+@pytest.mark.parametrize("per_range", [0, 64])
+@pytest.mark.parametrize("heads, kv_heads, dim, vdim, chunk", [
+    (4, 1, 64, 32, 44), (8, 2, 32, 64, 16), (6, 3, 64, 32, 0), (32, 2, 64, 64, 100), (2, 2, 128, 128, 7), (4, 2, 64, 64, 1)])
+def test_chunked_attention_on_the_matrix_cores_with_values_of_their_own_size(heads, kv_heads, dim, vdim, chunk, per_range, row_tiles, gpu):
+    page, scale, length = 16, 0.2, 200
+    assert K.attention_rows_mfma_supported(dim, vdim, page)
+    group = heads // kv_heads
+    q_all = rnd((length, heads, dim), 31).to(torch.bfloat16)
+    k_all, v_all = rnd((length, kv_heads, dim), 32).to(torch.bfloat16), rnd((length, kv_heads, vdim), 33).to(torch.bfloat16)
+    # a key that stands out for the last query of each entry below, at its chunk's first position or one before it
+    for qpos in (66, 199, 8, 112, 111):
+        first = (qpos // chunk) * chunk if chunk else 0
+        qf, kf = q_all.float(), k_all.float()
+        standout(qf, kf, qpos, max(0, first - (qpos % 2)), head=heads - 1, kv_head=kv_heads - 1, strength=14.0)
+        q_all, k_all = qf.to(torch.bfloat16), kf.to(torch.bfloat16)
+    table, slots, pages = cache_for(length, page, 19)
+    want_all = chunk_reference(q_all, k_all, v_all, scale, chunk)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")
+    for start, n in [(37, 30), (199, 1), (0, 9), (112, 1), (96, 16)]:
+        upto = start + n
+        kp = torch.full((pages, kv_heads, page, dim), float("nan"), dtype=torch.bfloat16, device="cuda")
+        v_cache = torch.full((pages, kv_heads, vdim, page), float("nan"), dtype=torch.bfloat16, device="cuda")
+        sl = slots[:upto].long().to("cuda")
+        kp[sl // page, :, sl % page] = k_all[:upto].to("cuda")
+        v_cache[sl // page, :, :, sl % page] = v_all[:upto].to("cuda")
+        k_cache = K.keys_to_pages(kp)
+        q = q_all[start:upto].reshape(n, heads * dim).contiguous().to("cuda")
+        per_item = 16 * row_tiles
+        tiles = (n * group + per_item - 1) // per_item
+        out = torch.empty((n, heads * vdim), dtype=torch.bfloat16, device="cuda")
+        ranges = 1 if per_range == 0 else -(-upto // per_range)
+        K.attention_rows_mfma(q, heads * dim, out, k_cache, v_cache, table.to("cuda"), i32([0] * tiles),
+                              i32([per_item * t for t in range(tiles)]), i32([1]), i32([0, n]), i32([start]), heads, kv_heads,
+                              dim, scale, 0, 0, None, vdim, ranges, per_range, row_tiles, chunk)
+        assert torch.isfinite(out.float()).all(), f"entry {start}+{n}"
+        torch.testing.assert_close(out.view(n, heads, vdim).cpu().to(F), want_all[start:upto], rtol=4e-2, atol=4e-2)
