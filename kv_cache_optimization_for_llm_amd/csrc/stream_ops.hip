@@ -202,11 +202,97 @@ norm_into_stream_kernel(void *__restrict__ x, int x_dtype, const void *__restric
     }
 }
 
+// The same for the shapes a bf16 engine with a 32-bit stream has (x fp32, y bf16, copy bf16 or none, a
+// width that is a multiple of 8 up to 2,048 * ITERS): a thread keeps its 8 * ITERS elements of y, x and w
+// in registers, all loads are asked for before the sum of squares is taken, and rows move 16 bytes a
+// lane.  At a few rows the launch is as long as its chain of trips to memory; this makes it one trip.
+template <int ITERS>
+__global__ void __launch_bounds__(256)
+norm_into_stream_vec_kernel(float *__restrict__ x, const uint16_t *__restrict__ y, const void *__restrict__ w, int w_dtype,
+                            uint16_t *__restrict__ copy, int width, float eps) {
+    __shared__ float red_s[4];
+    const size_t at = (size_t)blockIdx.x * width;
+    float yv[ITERS][8], xv[ITERS][8], wv[ITERS][8];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int j = (threadIdx.x + it * 256) * 8;
+        if (j < width) {
+            const uint4 yb = *reinterpret_cast<const uint4 *>(y + at + j);
+            const float4 x0 = *reinterpret_cast<const float4 *>(x + at + j), x1 = *reinterpret_cast<const float4 *>(x + at + j + 4);
+            const uint32_t yw[4] = {yb.x, yb.y, yb.z, yb.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                yv[it][2 * e] = __uint_as_float(yw[e] << 16);
+                yv[it][2 * e + 1] = __uint_as_float(yw[e] & 0xffff0000u);
+            }
+            xv[it][0] = x0.x; xv[it][1] = x0.y; xv[it][2] = x0.z; xv[it][3] = x0.w;
+            xv[it][4] = x1.x; xv[it][5] = x1.y; xv[it][6] = x1.z; xv[it][7] = x1.w;
+            if (w_dtype == KVA_F32) {
+                const float4 w0 = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(w) + j),
+                             w1 = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(w) + j + 4);
+                wv[it][0] = w0.x; wv[it][1] = w0.y; wv[it][2] = w0.z; wv[it][3] = w0.w;
+                wv[it][4] = w1.x; wv[it][5] = w1.y; wv[it][6] = w1.z; wv[it][7] = w1.w;
+            } else {
+                const uint4 wb = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(w) + j);
+                const uint32_t ww[4] = {wb.x, wb.y, wb.z, wb.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    wv[it][2 * e] = __uint_as_float(ww[e] << 16);
+                    wv[it][2 * e + 1] = __uint_as_float(ww[e] & 0xffff0000u);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) yv[it][e] = xv[it][e] = wv[it][e] = 0.f;
+        }
+    }
+    float sq = 0.f;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sq += yv[it][e] * yv[it][e];
+    const float inv = 1.0f / sqrtf(block_sum(sq, red_s, 4) / (float)width + eps);
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int j = (threadIdx.x + it * 256) * 8;
+        if (j >= width) continue;
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = xv[it][e] + yv[it][e] * inv * wv[it][e];
+        *reinterpret_cast<float4 *>(x + at + j) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4 *>(x + at + j + 4) = make_float4(v[4], v[5], v[6], v[7]);
+        if (copy) {
+            uint32_t c[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                c[e] = (uint32_t)float_to_bf16_bits(v[2 * e]) | ((uint32_t)float_to_bf16_bits(v[2 * e + 1]) << 16);
+            *reinterpret_cast<uint4 *>(copy + at + j) = make_uint4(c[0], c[1], c[2], c[3]);
+        }
+    }
+}
+
+static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
 extern "C" int kva_norm_into_stream(void *x, int x_dtype, const void *y, int y_dtype, const void *w, int w_dtype,
                                     void *copy, int copy_dtype, int rows, int width, float eps, hipStream_t stream) {
     KVA_REQUIRE(rows >= 0 && width > 0 && width <= 16000, "norm_into_stream: width %d must lie in 1..16000", width);
     KVA_REQUIRE(x && y && w && eps >= 0.f, "norm_into_stream: missing operand or negative eps");
     if (rows == 0) return KVA_OK;
+    // (which kernel runs depends on types and width alone, never on the rows: a row's numbers are the same in any batch)
+    if (x_dtype == KVA_F32 && y_dtype == KVA_BF16 && (!copy || copy_dtype == KVA_BF16) && width % 8 == 0 && width <= 8192 &&
+        aligned16(x) && aligned16(y) && aligned16(w) && aligned16(copy)) {
+        if (width <= 2048)
+            hipLaunchKernelGGL(norm_into_stream_vec_kernel<1>, dim3(rows), dim3(256), 0, stream, (float *)x, (const uint16_t *)y,
+                               w, w_dtype, (uint16_t *)copy, width, eps);
+        else if (width <= 4096)
+            hipLaunchKernelGGL(norm_into_stream_vec_kernel<2>, dim3(rows), dim3(256), 0, stream, (float *)x, (const uint16_t *)y,
+                               w, w_dtype, (uint16_t *)copy, width, eps);
+        else
+            hipLaunchKernelGGL(norm_into_stream_vec_kernel<4>, dim3(rows), dim3(256), 0, stream, (float *)x, (const uint16_t *)y,
+                               w, w_dtype, (uint16_t *)copy, width, eps);
+        KVA_CHECK_LAUNCH("norm_into_stream");
+        return KVA_OK;
+    }
     hipLaunchKernelGGL(norm_into_stream_kernel, dim3(rows), dim3(256), (size_t)width * sizeof(float), stream, x, x_dtype,
                        y, y_dtype, w, w_dtype, copy, copy_dtype, width, eps);
     KVA_CHECK_LAUNCH("norm_into_stream");

@@ -75,6 +75,26 @@ def test_gated_experts_against_the_plain_mixture(width, ff, experts, top, shared
     torch.testing.assert_close(got.cpu().to(F), want, **tol)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width", [4, 50, 72, 2048, 2050])                      # multiples of four move 16 bytes a lane
+def test_weighted_sum_with_identity_choices_and_one_more_addend(width, dtype, gpu):
+    T, top, experts = 13, 3, 5
+    g = torch.Generator().manual_seed(width)
+    x, extra = (torch.randn(T, width, generator=g).to(dtype) for _ in range(2))
+    rows = torch.randn(T * top, width, generator=g)
+    idx = torch.randint(0, experts + 2, (T, top), generator=g)                   # choices past the experts return the token itself
+    wgt = torch.rand(T, top, generator=g)
+    for more in (None, extra):
+        out = torch.empty((T, width), dtype=dtype, device="cuda")
+        K.moe_combine(dev(x, dtype), dev(rows), dev(idx, torch.int32), dev(wgt), experts, out, extra=None if more is None else dev(more, dtype))
+        real = (idx < experts)[:, :, None].to(F)
+        want = (real * rows.view(T, top, width).to(F) + (1 - real) * wgt[:, :, None].to(F) * x.to(F)[:, None, :]).sum(1)
+        if more is not None:
+            want = want + more.to(F)
+        tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-2, atol=2e-2)
+        torch.testing.assert_close(out.cpu().to(F), want, **tol)
+
+
 # ---- one fixed decay a head ------------------------------------------------------------------------
 @pytest.mark.parametrize("heads, dim, vdim", [(4, 48, 32), (1, 16, 16), (3, 20, 9), (2, 128, 40), (5, 8, 64), (2, 144, 18), (1, 100, 5)])
 @pytest.mark.parametrize("portions", [(1000,), (1,), (3, 1, 16, 2, 50), (31, 33, 32, 1)])
@@ -212,19 +232,20 @@ def test_a_far_token_under_a_decay_of_one_and_a_seat_taken_again(gpu):
 
 
 # ---- a branch's output normed on its way into the stream -----------------------------------------
-@pytest.mark.parametrize("width", [8, 72, 96, 256, 2048, 4104])
-@pytest.mark.parametrize("stream, branch, copy", [("float32", "float32", None), ("float32", "bfloat16", "bfloat16"),
-                                                 ("float32", "bfloat16", None), ("bfloat16", "bfloat16", "bfloat16"),
-                                                 ("float32", "float32", "float32")])
-def test_norm_into_stream(width, stream, branch, copy, gpu):
+@pytest.mark.parametrize("width", [8, 72, 96, 100, 256, 2048, 2056, 4104, 8200])      # (multiples of 8 up to 8,192 have a kernel of their own)
+@pytest.mark.parametrize("stream, branch, copy, weight", [
+    ("float32", "float32", None, "float32"), ("float32", "bfloat16", "bfloat16", "bfloat16"), ("float32", "bfloat16", None, "float32"),
+    ("float32", "bfloat16", "bfloat16", "float32"), ("bfloat16", "bfloat16", "bfloat16", "bfloat16"),
+    ("float32", "float32", "float32", "float32"), ("float32", "bfloat16", "float32", "bfloat16")])
+def test_norm_into_stream(width, stream, branch, copy, weight, gpu):
     T, eps = 19, 0.01
     x = rnd((T, width), width, 3.0).to(DT[stream])
     y = rnd((T, width), width + 1, 0.5).to(DT[branch])
     y[3] = 0.0                                               # a row of zeros stays zero: eps stands inside the root
-    w = (rnd((width,), width + 2, 0.3) + 1.0).to(DT[branch])
+    w = (rnd((width,), width + 2, 0.3) + 1.0).to(DT[weight])
     xs = dev(x, DT[stream])
     cp = None if copy is None else torch.full((T, width), 7.0, dtype=DT[copy], device="cuda")
-    K.norm_into_stream(xs, dev(y, DT[branch]), dev(w, DT[branch]), eps, cp)
+    K.norm_into_stream(xs, dev(y, DT[branch]), dev(w, DT[weight]), eps, cp)
     want = x.to(F) + plain.rms_norm(y.to(F), w.to(F), eps)
     tol = dict(rtol=1e-5, atol=1e-5) if stream == "float32" else dict(rtol=1e-2, atol=2e-2)
     torch.testing.assert_close(xs.cpu().to(F), want, **tol)
