@@ -21,6 +21,7 @@ absent.  The model's norm at the end, logits from the token table itself, then a
 """
 from __future__ import annotations
 
+import copy
 from dataclasses import dataclass
 from typing import Any, Mapping, Optional, Tuple
 
@@ -46,6 +47,12 @@ def _kv_heads(m: Mapping[str, Any], where: str) -> None:
 
 
 def _check_mixer(kind: str, m: Mapping[str, Any], where: str, index: int, layers) -> None:
+    if kind == "attention" and isinstance(m, dict) and isinstance(m.get("kv_from"), int) and 0 <= m["kv_from"] < index:
+        # sizes of keys and values that such a layer leaves out are those of the layer it takes them from
+        om = layers[m["kv_from"]].get("mixer") if isinstance(layers[m["kv_from"]], Mapping) else None
+        for key in ("kv_heads", "dim", "vdim"):
+            if key not in m and isinstance(om, Mapping) and key in om:
+                m[key] = om[key]
     _positive(m, ("heads", "dim", "vdim"), where)
     if kind == "lightning":
         decay = m.get("decay")
@@ -110,6 +117,7 @@ class LomodraConfig:
         layers = d.get("layers")
         if not isinstance(layers, (list, tuple)) or not layers:
             raise ConfigError("config.json: 'layers' must be a non-empty list")
+        layers = copy.deepcopy(list(layers))      # (sizes a layer inherits are filled in below; the caller's dict stays)
         for i, layer in enumerate(layers):
             where = f"layers[{i}]"
             if not isinstance(layer, Mapping) or layer.get("type") not in LAYER_TYPES:

@@ -67,6 +67,17 @@ def test_tensor_names_and_shapes():
     assert specs["l3.mix.a1"].shape == (None, 96) and specs["l3.mix.g2"].shape == (96, None)
 
 
+def test_a_layer_that_names_no_key_and_value_sizes_takes_those_of_the_layer_it_reads():
+    cfg = copy.deepcopy(U.CFG_A)
+    for key in ("kv_heads", "dim", "vdim"):
+        del cfg["layers"][2]["mixer"][key]
+    before = copy.deepcopy(cfg)
+    assert tensor_specs_for_config(cfg) == tensor_specs_for_config(U.CFG_A) and cfg == before
+    del cfg["layers"][2]["mixer"]["heads"]
+    with pytest.raises(ConfigError, match="heads"):
+        spec_for_config(cfg)
+
+
 @pytest.mark.parametrize("edit, message", [
     (lambda c: c["layers"][0].update(type="conv"), "type"),
     (lambda c: c["layers"][0]["mixer"].update(kv_heads=3), "multiple"),
