@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 def random_config(seed: int) -> dict:
     rng = np.random.default_rng(seed)
     pick = lambda *xs: xs[int(rng.integers(len(xs)))]
-    width = pick(64, 72, 96, 100, 128, 160, 256, 320)
+    width = pick(64, 72, 96, 100, 128, 160, 192, 256)
 
     def mlp():
         if rng.random() < 0.2:
@@ -48,10 +48,10 @@ def random_config(seed: int) -> dict:
                 owners.append(len(layers))
                 layers.append(U.attention_layer(kv * pick(1, 2, 4), kv, dim, pick(dim, 16, 32, 64), pick(0.08, 0.125, 0.3),
                                                 chunk, mlp=mlp()))
-    cfg = {"architecture": "Lomodra", "vocab": pick(64, 101, 256, 333, 448), "width": width,
+    cfg = {"architecture": "Lomodra", "vocab": pick(64, 101, 256, 333, 400), "width": width,
            "norm": {"eps": pick(0.02, 0.05, 0.1)}, "layers": layers}
     if rng.random() < 0.8:
-        cfg["logit_softcap"] = float(pick(5.0, 15.0, 30.0))
+        cfg["logit_softcap"] = float(pick(5.0, 12.0, 30.0))
     if rng.random() < 0.8:
         cfg["token_side"] = {"dim": pick(1, 4, 12, 16, 32)}
     return cfg
