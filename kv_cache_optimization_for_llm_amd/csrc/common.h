@@ -178,11 +178,23 @@ enum KvaDtype { KVA_F32 = 0, KVA_BF16 = 1 };
 
 // Activations of a gated feed-forward, act(gate) * up: silu z / (1 + e^-z), relu, and the tanh
 // form of gelu, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))).
-enum KvaActivation { KVA_ACT_SILU = 0, KVA_ACT_RELU = 1, KVA_ACT_GELU_TANH = 2 };
+enum KvaActivation { KVA_ACT_SILU = 0, KVA_ACT_RELU = 1, KVA_ACT_GELU_TANH = 2, KVA_ACT_SWISH_CLAMPED = 3 };
 
 __device__ inline float kva_activate(float z, int act) {
     if (act == KVA_ACT_RELU) return z > 0.f ? z : 0.f;
     if (act == KVA_ACT_GELU_TANH)
         return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
     return z * (1.f / (1.f + expf(-z)));
+}
+
+// act(gate) * up of a gated feed-forward.  KVA_ACT_SWISH_CLAMPED is the clamped form: with g = min(gate,
+// limit) and u = clamp(up, -limit, limit) it is g * sigmoid(1.702 g) * (u + 1); the other activations
+// take no limit.
+#define KVA_SWISH_ALPHA 1.702f
+__device__ inline float kva_gated_activate(float gate, float up, int act, float limit) {
+    if (act == KVA_ACT_SWISH_CLAMPED) {
+        const float g = fminf(gate, limit), u = fminf(fmaxf(up, -limit), limit);
+        return g * (1.f / (1.f + expf(-KVA_SWISH_ALPHA * g))) * (u + 1.f);
+    }
+    return kva_activate(gate, act) * up;
 }

@@ -4,7 +4,7 @@
 //  * kva_qk_encode_cache: heads of queries and keys whose first `rot` elements are rotated with
 //    either pairing (pair i = elements (i, i + rot/2) or (2i, 2i + 1)), optionally followed by a
 //    division of every head by its root mean square (and a multiplication by a weight per element,
-//    one for queries and one for keys: an RMS norm of every head); keys of `head_dim` and values of another
+//    one for queries and one for keys: an RMS norm of every head) - or, with norm_first, preceded by it; keys of `head_dim` and values of another
 //    size `value_dim` go to the paged K / V^T arrays (kv_layout.h).
 //  * kva_latent_encode_cache: a low-rank key/value entry.  Per token one latent vector of `rank`
 //    elements, RMS-normed with a weight, and one rotated key part of `rot` elements shared by all
@@ -26,7 +26,7 @@ qk_encode_cache_kernel(T *__restrict__ qkv, int row_stride, int k_off, int v_off
                        const int *__restrict__ slot_mapping, int num_q_heads, int num_kv_heads, int head_dim,
                        int value_dim, int rot, int interleaved, float unit_eps, int page_size,
                        const T *__restrict__ bias, const float *__restrict__ q_weight,
-                       const float *__restrict__ k_weight) {
+                       const float *__restrict__ k_weight, int norm_first) {
     const int t = blockIdx.x;
     const int lane = threadIdx.x % KVA_WAVE, wave = threadIdx.x / KVA_WAVE, waves = blockDim.x / KVA_WAVE;
     T *row = qkv + (size_t)t * row_stride;
@@ -65,7 +65,7 @@ qk_encode_cache_kernel(T *__restrict__ qkv, int row_stride, int k_off, int v_off
             }
             const float u = to_float(h[i1[c]]) + (hb ? to_float(hb[i1[c]]) : 0.f);
             const float v = to_float(h[i2[c]]) + (hb ? to_float(hb[i2[c]]) : 0.f);
-            if (p < half) {
+            if (p < half && !norm_first) {
                 const float co = cs[p], si = sn[p];
                 o1[c] = u * co - v * si;
                 o2[c] = v * co + u * si;
@@ -86,7 +86,13 @@ qk_encode_cache_kernel(T *__restrict__ qkv, int row_stride, int k_off, int v_off
         for (int c = 0; c < PER; ++c) {
             const int p = lane + c * KVA_WAVE;
             if (p >= pairs) continue;
-            const T r1 = from_float<T>(o1[c] * mul * (nw ? nw[i1[c]] : 1.f)), r2 = from_float<T>(o2[c] * mul * (nw ? nw[i2[c]] : 1.f));
+            float f1 = o1[c] * mul * (nw ? nw[i1[c]] : 1.f), f2 = o2[c] * mul * (nw ? nw[i2[c]] : 1.f);
+            if (norm_first && p < half) {           // the normed head is what is rotated
+                const float co = cs[p], si = sn[p], u = f1, v = f2;
+                f1 = u * co - v * si;
+                f2 = v * co + u * si;
+            }
+            const T r1 = from_float<T>(f1), r2 = from_float<T>(f2);
             if (is_q) {
                 h[i1[c]] = r1;
                 h[i2[c]] = r2;
@@ -181,7 +187,9 @@ extern "C" int kva_qk_encode_cache(void *qkv, int row_stride, int k_off, int v_o
                                    const int *slot_mapping, int tokens, int num_q_heads, int num_kv_heads,
                                    int head_dim, int value_dim, int rot, int interleaved, float unit_eps,
                                    int page_size, int dtype, const void *bias, const float *q_weight,
-                                   const float *k_weight, hipStream_t stream) {
+                                   const float *k_weight, int norm_first, hipStream_t stream) {
+    // norm_first: the division by the root mean square (and the weight) comes before the rotation
+    KVA_REQUIRE(!norm_first || unit_eps >= 0.f, "qk_encode_cache: a norm before the rotation needs the norm");
     // (num_kv_heads = 0: rows of queries alone, for a layer that reads another layer's keys and values)
     KVA_REQUIRE(tokens >= 0 && num_q_heads > 0 && num_kv_heads >= 0 && value_dim > 0, "qk_encode_cache: bad sizes");
     KVA_REQUIRE(num_kv_heads > 0 || !slot_mapping, "qk_encode_cache: a cache write without key heads");
@@ -199,7 +207,7 @@ extern "C" int kva_qk_encode_cache(void *qkv, int row_stride, int k_off, int v_o
     if (tokens == 0) return KVA_OK;
     if (rot == 0) cos_table = sin_table = reinterpret_cast<const float *>(qkv);     // never read
     const int vecs = head_dim / 8;
-    if (!bias && !q_weight && !k_weight && dtype == KVA_BF16 && interleaved && head_dim % 8 == 0 && (vecs & (vecs - 1)) == 0 && vecs <= KVA_WAVE &&
+    if (!bias && !q_weight && !k_weight && !norm_first && dtype == KVA_BF16 && interleaved && head_dim % 8 == 0 && (vecs & (vecs - 1)) == 0 && vecs <= KVA_WAVE &&
         row_stride % 8 == 0 && k_off % 8 == 0 && (reinterpret_cast<uintptr_t>(qkv) & 15) == 0) {
         hipLaunchKernelGGL(qk_encode_cache_vec_kernel, dim3(tokens), dim3(256), 0, stream, (bf16_t *)qkv, row_stride,
                            k_off, v_off, (bf16_t *)k_cache, (bf16_t *)v_cache, cos_table, sin_table, positions,
@@ -211,12 +219,12 @@ extern "C" int kva_qk_encode_cache(void *qkv, int row_stride, int k_off, int v_o
         hipLaunchKernelGGL(qk_encode_cache_kernel<float>, dim3(tokens), dim3(256), 0, stream, (float *)qkv, row_stride,
                            k_off, v_off, (float *)k_cache, (float *)v_cache, cos_table, sin_table, positions,
                            slot_mapping, num_q_heads, num_kv_heads, head_dim, value_dim, rot, interleaved, unit_eps,
-                           page_size, (const float *)bias, q_weight, k_weight);
+                           page_size, (const float *)bias, q_weight, k_weight, norm_first);
     else if (dtype == KVA_BF16)
         hipLaunchKernelGGL(qk_encode_cache_kernel<bf16_t>, dim3(tokens), dim3(256), 0, stream, (bf16_t *)qkv,
                            row_stride, k_off, v_off, (bf16_t *)k_cache, (bf16_t *)v_cache, cos_table, sin_table,
                            positions, slot_mapping, num_q_heads, num_kv_heads, head_dim, value_dim, rot, interleaved,
-                           unit_eps, page_size, (const bf16_t *)bias, q_weight, k_weight);
+                           unit_eps, page_size, (const bf16_t *)bias, q_weight, k_weight, norm_first);
     else KVA_REQUIRE(false, "qk_encode_cache: unsupported dtype %d", dtype);
     KVA_CHECK_LAUNCH("qk_encode_cache");
     return KVA_OK;

@@ -36,10 +36,13 @@ __device__ inline float moe_activate(float z, int act) {
 __global__ void __launch_bounds__(256)
 moe_route_kernel(int *__restrict__ idx, float *__restrict__ wgt, const float *__restrict__ logits,
                  const float *__restrict__ correction, int tokens, int outputs, int top, int renormalise,
-                 int over_chosen) {
+                 int over_chosen, int sigmoid_scores, int groups, int keep_groups, int group_top, float weight_scale,
+                 float sum_eps) {
+    __shared__ float choice_s[4][KVA_WAVE * MOE_ROUTE_PER_LANE];
     const int lane = threadIdx.x % KVA_WAVE;
     const int t = blockIdx.x * (blockDim.x / KVA_WAVE) + threadIdx.x / KVA_WAVE;
     if (t >= tokens) return;
+    float *choice = choice_s[threadIdx.x / KVA_WAVE];
     float s[MOE_ROUTE_PER_LANE], ch[MOE_ROUTE_PER_LANE];
     float mx = -INFINITY;
 #pragma unroll
@@ -65,8 +68,54 @@ moe_route_kernel(int *__restrict__ idx, float *__restrict__ wgt, const float *__
             // alone: exp(logit - max) here, divided by the chosen ones' sum below
             ch[j] = e < outputs ? logits[(size_t)t * outputs + e] + (correction ? correction[e] : 0.f) : -INFINITY;
         } else {
-            s[j] = s[j] / sum;
+            // scores: the softmax over all outputs, or every output's own sigmoid
+            s[j] = sigmoid_scores ? (e < outputs ? 1.f / (1.f + expf(-logits[(size_t)t * outputs + e])) : 0.f) : s[j] / sum;
             ch[j] = e < outputs ? s[j] + (correction ? correction[e] : 0.f) : -INFINITY;
+        }
+    }
+    if (groups > 1) {
+        // Outputs form `groups` equal runs of neighbours.  A group's score is the sum of its `group_top`
+        // largest choice scores; only outputs of the `keep_groups` best groups (of equal ones the lowest
+        // index) can be chosen: the others' choice scores become -inf.  Lane g takes group g.
+        const int per = outputs / groups;
+#pragma unroll
+        for (int j = 0; j < MOE_ROUTE_PER_LANE; ++j)
+            if (lane + j * KVA_WAVE < outputs) choice[lane + j * KVA_WAVE] = ch[j];
+        __builtin_amdgcn_wave_barrier();
+        __threadfence_block();
+        float gs = -INFINITY;
+        if (lane < groups) {
+            gs = 0.f;
+            unsigned long long taken = 0ull;            // (a group holds at most 64 outputs when it is scored this way; larger ones below)
+            for (int k = 0; k < group_top && k < per; ++k) {
+                float bv = -INFINITY;
+                int bi = -1;
+                for (int i = 0; i < per; ++i) {
+                    const bool used = i < 64 ? ((taken >> i) & 1ull) != 0ull : false;
+                    const float v = choice[lane * per + i];
+                    if (!used && (bi < 0 || v > bv)) { bv = v; bi = i; }
+                }
+                if (bi >= 0 && bi < 64) taken |= 1ull << bi;
+                gs += bv;
+            }
+        }
+        unsigned long long allowed = 0ull;
+        for (int k = 0; k < keep_groups; ++k) {
+            float bv = gs;
+            int bg = lane < groups && !((allowed >> lane) & 1ull) ? lane : 0x7fffffff;
+            if (bg == 0x7fffffff) bv = -INFINITY;
+#pragma unroll
+            for (int off = KVA_WAVE / 2; off > 0; off >>= 1) {
+                const float ov = __shfl_xor(bv, off, KVA_WAVE);
+                const int og = __shfl_xor(bg, off, KVA_WAVE);
+                if (og != 0x7fffffff && (bg == 0x7fffffff || ov > bv || (ov == bv && og < bg))) { bv = ov; bg = og; }
+            }
+            if (bg != 0x7fffffff) allowed |= 1ull << bg;
+        }
+#pragma unroll
+        for (int j = 0; j < MOE_ROUTE_PER_LANE; ++j) {
+            const int e = lane + j * KVA_WAVE;
+            if (e < outputs && !((allowed >> (e / per)) & 1ull)) ch[j] = -INFINITY;
         }
     }
     float total = 0.f;
@@ -94,19 +143,32 @@ moe_route_kernel(int *__restrict__ idx, float *__restrict__ wgt, const float *__
             wgt[(size_t)t * top + k] = bs;
         }
     }
-    if ((renormalise || over_chosen) && lane == 0)
-        for (int k = 0; k < top; ++k) wgt[(size_t)t * top + k] /= total;
+    if (lane == 0) {
+        if (renormalise || over_chosen)
+            for (int k = 0; k < top; ++k) wgt[(size_t)t * top + k] = wgt[(size_t)t * top + k] / (total + sum_eps) * weight_scale;
+        else if (weight_scale != 1.f)
+            for (int k = 0; k < top; ++k) wgt[(size_t)t * top + k] *= weight_scale;
+    }
 }
 
 extern "C" int kva_moe_route(int *idx, float *wgt, const float *logits, const float *correction, int tokens,
-                             int outputs, int top, int renormalise, int over_chosen, hipStream_t stream) {
+                             int outputs, int top, int renormalise, int over_chosen, int sigmoid_scores, int groups,
+                             int keep_groups, int group_top, float weight_scale, float sum_eps, hipStream_t stream) {
+    KVA_REQUIRE(groups >= 1 && groups <= KVA_WAVE && outputs % groups == 0 && keep_groups >= 1 && keep_groups <= groups &&
+                    group_top >= 1,
+                "moe_route: %d groups (at most %d, dividing the %d outputs) of which %d are kept", groups, KVA_WAVE, outputs,
+                keep_groups);
+    KVA_REQUIRE(groups == 1 || (outputs / groups <= 64 && top <= keep_groups * (outputs / groups)),
+                "moe_route: groups of at most 64 outputs, and enough outputs in the kept groups for top %d", top);
+    KVA_REQUIRE(!(sigmoid_scores && over_chosen), "moe_route: sigmoid scores exclude the softmax over the chosen logits");
     KVA_REQUIRE(idx && wgt && logits && tokens >= 0, "moe_route: missing operand");
     KVA_REQUIRE(outputs > 0 && outputs <= KVA_WAVE * MOE_ROUTE_PER_LANE, "moe_route: %d router outputs (at most %d)",
                 outputs, KVA_WAVE * MOE_ROUTE_PER_LANE);
     KVA_REQUIRE(top > 0 && top <= outputs, "moe_route: top %d of %d", top, outputs);
     if (tokens == 0) return KVA_OK;
     hipLaunchKernelGGL(moe_route_kernel, dim3((tokens + 3) / 4), dim3(256), 0, stream, idx, wgt, logits, correction,
-                       tokens, outputs, top, renormalise, over_chosen);
+                       tokens, outputs, top, renormalise, over_chosen, sigmoid_scores, groups, keep_groups, group_top,
+                       weight_scale, sum_eps);
     KVA_CHECK_LAUNCH("moe_route");
     return KVA_OK;
 }
@@ -161,11 +223,12 @@ struct MoeRows {
     const float *slot_weight;       // mode 1
     int top, N, K, mode, act;
     int gated;                      // mode 0: rows 2 j and 2 j + 1 of the matrix are output j's gate and up rows
+    float limit;                    // activation 4 (clamped swish): gate and up are cut off at this value
 };
 
 // mode 0 of a gated expert: outputs n (even) and n + 1 of the product are one output of the layer
 __device__ inline void moe_store_gated(const MoeRows &a, void *out, int out_dtype, int place, int n, float gate, float up) {
-    const float v = moe_activate(gate, a.act) * up;
+    const float v = a.act == 4 ? kva_gated_activate(gate, up, KVA_ACT_SWISH_CLAMPED, a.limit) : moe_activate(gate, a.act) * up;
     const size_t at = (size_t)place * (a.N / 2) + n / 2;
     if (out_dtype == KVA_BF16) reinterpret_cast<uint16_t *>(out)[at] = float_to_bf16_bits(v);
     else reinterpret_cast<float *>(out)[at] = v;
@@ -330,17 +393,18 @@ moe_expert_rows_mfma_kernel(MoeRows a, void *__restrict__ out, int out_dtype, co
 
 extern "C" int kva_moe_expert_rows(void *out, int out_dtype, const void *x, const void *w, int dtype,
                                    const int *sorted_slot, const int *tile_expert, const float *slot_weight,
-                                   int max_tiles, int top, int N, int K, int mode, int act, int gated,
+                                   int max_tiles, int top, int N, int K, int mode, int act, int gated, float limit,
                                    hipStream_t stream) {
+    KVA_REQUIRE(act != 4 || gated, "moe_expert_rows: the clamped activation is a gated one");
     KVA_REQUIRE(!gated || (mode == 0 && N % 2 == 0), "moe_expert_rows: gate and up rows come in pairs, in the first product");
     KVA_REQUIRE(out && x && w && sorted_slot && tile_expert, "moe_expert_rows: missing operand");
     KVA_REQUIRE(mode == 0 || (mode == 1 && slot_weight && out_dtype == KVA_F32),
                 "moe_expert_rows: mode 1 writes fp32 rows times a weight per slot");
     KVA_REQUIRE(mode == 1 || out_dtype == dtype, "moe_expert_rows: mode 0 writes rows of the operands' type");
-    KVA_REQUIRE(N > 0 && K > 0 && top > 0 && act >= 0 && act <= 3, "moe_expert_rows: bad sizes or activation");
+    KVA_REQUIRE(N > 0 && K > 0 && top > 0 && act >= 0 && act <= 4, "moe_expert_rows: bad sizes or activation");
     KVA_REQUIRE(max_tiles >= 0 && max_tiles <= 65535, "moe_expert_rows: %d tiles are too many for one launch", max_tiles);
     if (max_tiles == 0) return KVA_OK;
-    MoeRows a{sorted_slot, tile_expert, slot_weight, top, N, K, mode, act, gated};
+    MoeRows a{sorted_slot, tile_expert, slot_weight, top, N, K, mode, act, gated, limit};
     if (dtype == KVA_BF16 && K % 32 == 0) {
         // few tiles: 16 outputs a workgroup, so that enough of them stream the matrices; many: 64 outputs and
         // four row tiles, which share what they load
@@ -369,9 +433,11 @@ __device__ inline float moe_ld(const void *p, int dtype, size_t i) {
 
 __global__ void __launch_bounds__(256)
 moe_combine_kernel(void *__restrict__ out, const void *__restrict__ x, int dtype, const float *__restrict__ rows,
-                   const int *__restrict__ idx, const float *__restrict__ wgt, const void *__restrict__ extra, int width,
-                   int top, int experts) {
+                   const int *__restrict__ idx, const float *__restrict__ wgt, const void *__restrict__ extra,
+                   const float *__restrict__ extra_gate, int width, int top, int experts) {
     const size_t t = blockIdx.x;
+    // (optional) the addend enters times sigmoid(extra_gate[t]), one number a token
+    const float eg = extra && extra_gate ? 1.f / (1.f + expf(-extra_gate[t])) : 1.f;
     if (width % 4 == 0 && ((reinterpret_cast<uintptr_t>(rows) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
         // four neighbouring columns a thread, 16 bytes of every row at a time; the additions per column are
         // in the order of the scalar loop below
@@ -390,7 +456,7 @@ moe_combine_kernel(void *__restrict__ out, const void *__restrict__ x, int dtype
             }
             if (extra) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) acc[e] += moe_ld(extra, dtype, t * width + j + e);
+                for (int e = 0; e < 4; ++e) acc[e] += eg * moe_ld(extra, dtype, t * width + j + e);
             }
             if (dtype == KVA_BF16) {
                 const uint2 o = make_uint2((uint32_t)float_to_bf16_bits(acc[0]) | ((uint32_t)float_to_bf16_bits(acc[1]) << 16),
@@ -411,21 +477,21 @@ moe_combine_kernel(void *__restrict__ out, const void *__restrict__ x, int dtype
                                                     : reinterpret_cast<const float *>(x)[t * width + j]);
         }
         // what an expert that every token uses returned, with weight 1
-        if (extra) acc += dtype == KVA_BF16 ? bf16_bits_to_float(reinterpret_cast<const uint16_t *>(extra)[t * width + j])
-                                            : reinterpret_cast<const float *>(extra)[t * width + j];
+        if (extra) acc += eg * (dtype == KVA_BF16 ? bf16_bits_to_float(reinterpret_cast<const uint16_t *>(extra)[t * width + j])
+                                                  : reinterpret_cast<const float *>(extra)[t * width + j]);
         if (dtype == KVA_BF16) reinterpret_cast<uint16_t *>(out)[t * width + j] = float_to_bf16_bits(acc);
         else reinterpret_cast<float *>(out)[t * width + j] = acc;
     }
 }
 
 extern "C" int kva_moe_combine(void *out, const void *x, int dtype, const float *rows, const int *idx,
-                               const float *wgt, const void *extra, int tokens, int width, int top, int experts,
-                               hipStream_t stream) {
+                               const float *wgt, const void *extra, const float *extra_gate, int tokens, int width,
+                               int top, int experts, hipStream_t stream) {
     KVA_REQUIRE(out && x && rows && idx && wgt && width > 0 && top > 0, "moe_combine: missing operand");
     KVA_REQUIRE(dtype == KVA_BF16 || dtype == KVA_F32, "moe_combine: unsupported dtype %d", dtype);
     if (tokens <= 0) return KVA_OK;
-    hipLaunchKernelGGL(moe_combine_kernel, dim3(tokens), dim3(256), 0, stream, out, x, dtype, rows, idx, wgt, extra, width,
-                       top, experts);
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(tokens), dim3(256), 0, stream, out, x, dtype, rows, idx, wgt, extra, extra_gate,
+                       width, top, experts);
     KVA_CHECK_LAUNCH("moe_combine");
     return KVA_OK;
 }

@@ -48,13 +48,15 @@ __device__ inline float rec_column_sum(float v) {
 }
 
 // ---- short causal convolution + silu -----------------------------------------------------
-// out[row, c] = silu(sum_j w[c, j] * in(row - taps + 1 + j)[c]); inputs before the step's first
+// out[row, c] = act(sum_j w[c, j] * in(row - taps + 1 + j)[c] + out_bias[c]) with act = silu or none and
+// in = y + in_bias (both biases optional); inputs before the step's first
 // token of the request come from the seat's state [channels, taps - 1] (slot taps - 2 newest).
 __global__ void __launch_bounds__(256)
 causal_conv_act_kernel(float *__restrict__ out, int out_stride, const void *__restrict__ y, int y_dtype, int y_stride,
                        int col_off, const void *__restrict__ w, int w_dtype, const float *__restrict__ state,
                        size_t seat_stride, int conv_off, const int *__restrict__ entry_q_start,
-                       const int *__restrict__ entry_seat, int channels, int taps, int tokens_per_block) {
+                       const int *__restrict__ entry_seat, int channels, int taps, int tokens_per_block,
+                       const float *__restrict__ in_bias, const float *__restrict__ out_bias, int act) {
     const int e = blockIdx.y;
     const int q0 = entry_q_start[e], n = entry_q_start[e + 1] - q0;
     const int first = blockIdx.x * tokens_per_block;
@@ -66,11 +68,13 @@ causal_conv_act_kernel(float *__restrict__ out, int out_stride, const void *__re
             float acc = 0.f;
             for (int j = 0; j < taps; ++j) {
                 const int src = i - (taps - 1) + j;
-                const float x = src >= 0 ? rec_ld(y, y_dtype, (size_t)(q0 + src) * y_stride + col_off + c)
+                // (the state holds inputs with their bias already added; before a request's start it holds zeros)
+                const float x = src >= 0 ? rec_ld(y, y_dtype, (size_t)(q0 + src) * y_stride + col_off + c) + (in_bias ? in_bias[c] : 0.f)
                                          : st[(size_t)c * (taps - 1) + (taps - 1) + src];
                 acc += rec_ld(w, w_dtype, (size_t)c * taps + j) * x;
             }
-            out[(size_t)(q0 + i) * out_stride + c] = rec_silu(acc);
+            if (out_bias) acc += out_bias[c];
+            out[(size_t)(q0 + i) * out_stride + c] = rec_act(acc, act);
         }
     }
 }
@@ -79,7 +83,7 @@ causal_conv_act_kernel(float *__restrict__ out, int out_stride, const void *__re
 __global__ void __launch_bounds__(256)
 conv_state_update_kernel(float *__restrict__ state, size_t seat_stride, int conv_off, const void *__restrict__ y,
                          int y_dtype, int y_stride, int col_off, const int *__restrict__ entry_q_start,
-                         const int *__restrict__ entry_seat, int channels, int taps) {
+                         const int *__restrict__ entry_seat, int channels, int taps, const float *__restrict__ in_bias) {
     const int e = blockIdx.y;
     const int q0 = entry_q_start[e], n = entry_q_start[e + 1] - q0;
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
@@ -88,7 +92,7 @@ conv_state_update_kernel(float *__restrict__ state, size_t seat_stride, int conv
     float keep[16];
     for (int s = 0; s < taps - 1; ++s) {
         const int src = n - (taps - 1) + s;
-        keep[s] = src >= 0 ? rec_ld(y, y_dtype, (size_t)(q0 + src) * y_stride + col_off + c) : st[s + n];
+        keep[s] = src >= 0 ? rec_ld(y, y_dtype, (size_t)(q0 + src) * y_stride + col_off + c) + (in_bias ? in_bias[c] : 0.f) : st[s + n];
     }
     for (int s = 0; s < taps - 1; ++s) st[s] = keep[s];
 }
@@ -96,7 +100,9 @@ conv_state_update_kernel(float *__restrict__ state, size_t seat_stride, int conv
 extern "C" int kva_causal_conv_act(float *out, int out_stride, const void *y, int y_dtype, int y_stride, int col_off,
                                    const void *w, int w_dtype, float *state, long long seat_stride, int conv_off,
                                    const int *entry_q_start, const int *entry_seat, int entries, int max_q_len,
-                                   int channels, int taps, hipStream_t stream) {
+                                   int channels, int taps, const float *in_bias, const float *out_bias, int act,
+                                   hipStream_t stream) {
+    KVA_REQUIRE(act == 0 || act == 1, "causal_conv_act: activation %d is neither none (0) nor silu (1)", act);
     KVA_REQUIRE(out && y && w && state && entry_q_start && entry_seat, "causal_conv_act: missing operand");
     KVA_REQUIRE(channels > 0 && taps >= 1 && taps <= 17, "causal_conv_act: taps %d must lie in 1..17", taps);
     KVA_REQUIRE(entries >= 0 && entries <= 65535 && max_q_len >= 0, "causal_conv_act: bad batch");
@@ -104,12 +110,12 @@ extern "C" int kva_causal_conv_act(float *out, int out_stride, const void *y, in
     const int per = 8;
     hipLaunchKernelGGL(causal_conv_act_kernel, dim3((max_q_len + per - 1) / per, entries), dim3(256), 0, stream, out,
                        out_stride, y, y_dtype, y_stride, col_off, w, w_dtype, state, (size_t)seat_stride, conv_off,
-                       entry_q_start, entry_seat, channels, taps, per);
+                       entry_q_start, entry_seat, channels, taps, per, in_bias, out_bias, act);
     KVA_CHECK_LAUNCH("causal_conv_act");
     if (taps > 1) {
         hipLaunchKernelGGL(conv_state_update_kernel, dim3((channels + 255) / 256, entries), dim3(256), 0, stream, state,
                            (size_t)seat_stride, conv_off, y, y_dtype, y_stride, col_off, entry_q_start, entry_seat,
-                           channels, taps);
+                           channels, taps, in_bias);
         KVA_CHECK_LAUNCH("conv_state_update");
     }
     return KVA_OK;
@@ -704,7 +710,7 @@ extern "C" int kva_gated_linear_attention(float *out, float *state, long long se
 __global__ void __launch_bounds__(256)
 head_norm_gate_kernel(void *__restrict__ out, int out_dtype, int out_stride, int out_off, const void *__restrict__ x,
                       int x_dtype, const float *__restrict__ w, float eps, const void *__restrict__ gate,
-                      int gate_dtype, int gate_stride, int gate_off, int heads, int dv, int act, float mul) {
+                      int gate_dtype, int gate_stride, int gate_off, int heads, int dv, int act, float mul, int w_stride) {
     const size_t t = blockIdx.x;
     const int lane = threadIdx.x % KVA_WAVE, wave = threadIdx.x / KVA_WAVE, waves = blockDim.x / KVA_WAVE;
     for (int h = wave; h < heads; h += waves) {
@@ -720,9 +726,12 @@ head_norm_gate_kernel(void *__restrict__ out, int out_dtype, int out_stride, int
         }
         for (int j = lane; j < dv; j += KVA_WAVE) {
             float v = rec_ld(x, x_dtype, base + j);
-            if (w) v = v * inv * w[j];
-            const float g = rec_ld(gate, gate_dtype, t * gate_stride + gate_off + h * dv + j);
-            v *= (act == 1 ? rec_sigmoid(g) : rec_silu(g)) * mul;
+            if (w) v = v * inv * w[(size_t)h * w_stride + j];
+            if (gate) {
+                const float g = rec_ld(gate, gate_dtype, t * gate_stride + gate_off + h * dv + j);
+                v *= (act == 1 ? rec_sigmoid(g) : rec_silu(g));
+            }
+            v *= mul;
             rec_st(out, out_dtype, t * out_stride + out_off + h * dv + j, v);
         }
     }
@@ -733,7 +742,7 @@ head_norm_gate_kernel(void *__restrict__ out, int out_dtype, int out_stride, int
 __global__ void __launch_bounds__(256)
 head_norm_gate_wide_kernel(void *__restrict__ out, int out_dtype, int out_stride, int out_off, const void *__restrict__ x,
                            int x_dtype, const float *__restrict__ w, float eps, const void *__restrict__ gate,
-                           int gate_dtype, int gate_stride, int gate_off, int heads, int dv, int act, float mul) {
+                           int gate_dtype, int gate_stride, int gate_off, int heads, int dv, int act, float mul, int w_stride) {
     __shared__ float red_s[4];
     const size_t t = blockIdx.x;
     for (int h = 0; h < heads; ++h) {
@@ -749,9 +758,12 @@ head_norm_gate_wide_kernel(void *__restrict__ out, int out_dtype, int out_stride
         }
         for (int j = threadIdx.x; j < dv; j += blockDim.x) {
             float v = rec_ld(x, x_dtype, base + j);
-            if (w) v = v * inv * w[j];
-            const float g = rec_ld(gate, gate_dtype, t * gate_stride + gate_off + h * dv + j);
-            v *= (act == 1 ? rec_sigmoid(g) : rec_silu(g)) * mul;
+            if (w) v = v * inv * w[(size_t)h * w_stride + j];
+            if (gate) {
+                const float g = rec_ld(gate, gate_dtype, t * gate_stride + gate_off + h * dv + j);
+                v *= (act == 1 ? rec_sigmoid(g) : rec_silu(g));
+            }
+            v *= mul;
             rec_st(out, out_dtype, t * out_stride + out_off + h * dv + j, v);
         }
     }
@@ -759,16 +771,265 @@ head_norm_gate_wide_kernel(void *__restrict__ out, int out_dtype, int out_stride
 
 extern "C" int kva_head_norm_gate(void *out, int out_dtype, int out_stride, int out_off, const void *x, int x_dtype,
                                   const float *w, float eps, const void *gate, int gate_dtype, int gate_stride,
-                                  int gate_off, int rows, int heads, int dv, int act, float mul, hipStream_t stream) {
-    KVA_REQUIRE(out && x && gate && heads > 0 && dv > 0 && rows >= 0, "head_norm_gate: missing operand or bad sizes");
+                                  int gate_off, int rows, int heads, int dv, int act, float mul, int w_stride,
+                                  hipStream_t stream) {
+    // w_stride: 0 - one weight of dv elements shared by the heads; dv - a weight of heads * dv elements.  gate may be absent.
+    KVA_REQUIRE(out && x && heads > 0 && dv > 0 && rows >= 0, "head_norm_gate: missing operand or bad sizes");
+    KVA_REQUIRE(w_stride == 0 || w_stride == dv, "head_norm_gate: a weight is shared by the heads or has all heads' size");
     KVA_REQUIRE(act == 0 || act == 1, "head_norm_gate: activation %d is neither silu (0) nor sigmoid (1)", act);
     if (rows == 0) return KVA_OK;
     if (heads < 4 && dv >= 256)
         hipLaunchKernelGGL(head_norm_gate_wide_kernel, dim3(rows), dim3(256), 0, stream, out, out_dtype, out_stride, out_off,
-                           x, x_dtype, w, eps, gate, gate_dtype, gate_stride, gate_off, heads, dv, act, mul);
+                           x, x_dtype, w, eps, gate, gate_dtype, gate_stride, gate_off, heads, dv, act, mul, w_stride);
     else
         hipLaunchKernelGGL(head_norm_gate_kernel, dim3(rows), dim3(256), 0, stream, out, out_dtype, out_stride, out_off, x,
-                           x_dtype, w, eps, gate, gate_dtype, gate_stride, gate_off, heads, dv, act, mul);
+                           x_dtype, w, eps, gate, gate_dtype, gate_stride, gate_off, heads, dv, act, mul, w_stride);
     KVA_CHECK_LAUNCH("head_norm_gate");
+    return KVA_OK;
+}
+
+// ---- a real-gated linear recurrent unit ------------------------------------------------------------
+// Channels come in `blocks` equal runs; inside run b two square matrices [out, in] make the gates from
+// the run's own inputs u_b: r = sigmoid(A_b u_b + a_b), i = sigmoid(B_b u_b + b_b).  The recurrence
+// S_t = a_t S_(t-1) + sqrt(1 - a_t^2) i_t u_t with log a_t = -rate_c r_t (rate_c = 8 softplus(lam_c), formed
+// once when the weights are loaded) is linear in S, so this kernel forms, for all tokens side by side,
+// a_t and the input b_t = sqrt(1 - a_t^2) i_t u_t, and kva_linear_scan_gate walks the tokens.
+// A workgroup takes 16 tokens x 64 outputs of one run; thread (row, cx) four neighbouring outputs.
+// k ascending: a token's numbers do not depend on the batch.
+__global__ void __launch_bounds__(256)
+block_gates_kernel(float *__restrict__ a_out, float *__restrict__ b_out, const float *__restrict__ u, int tokens, int width,
+                   int bs, const void *__restrict__ wa, const void *__restrict__ wi, int w_dtype,
+                   const float *__restrict__ ba, const float *__restrict__ bi, const float *__restrict__ rate) {
+    __shared__ float us[16][33], was[64][33], wis[64][33];
+    const int blk = blockIdx.y, t0 = blockIdx.z * 16, n0 = blockIdx.x * 64;
+    const int row = threadIdx.x / 16, cx = threadIdx.x % 16;
+    const size_t wbase = (size_t)blk * bs * bs;
+    float ar[4] = {0.f, 0.f, 0.f, 0.f}, ai[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < bs; k0 += 32) {
+        __syncthreads();
+        for (int i = threadIdx.x; i < 16 * 32; i += 256) {
+            const int rr = i / 32, kk = k0 + i % 32;
+            us[rr][i % 32] = (t0 + rr < tokens && kk < bs) ? u[(size_t)(t0 + rr) * width + blk * bs + kk] : 0.f;
+        }
+        for (int i = threadIdx.x; i < 64 * 32; i += 256) {
+            const int nn = n0 + i / 32, kk = k0 + i % 32;
+            const bool in = nn < bs && kk < bs;
+            was[i / 32][i % 32] = in ? rec_ld(wa, w_dtype, wbase + (size_t)nn * bs + kk) : 0.f;
+            wis[i / 32][i % 32] = in ? rec_ld(wi, w_dtype, wbase + (size_t)nn * bs + kk) : 0.f;
+        }
+        __syncthreads();
+        for (int kk = 0; kk < 32; ++kk) {
+            const float xv = us[row][kk];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                ar[j] += xv * was[4 * cx + j][kk];
+                ai[j] += xv * wis[4 * cx + j][kk];
+            }
+        }
+    }
+    const int t = t0 + row;
+    if (t >= tokens) return;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int n = n0 + 4 * cx + j;
+        if (n >= bs) continue;
+        const int c = blk * bs + n;
+        const float r = rec_sigmoid(ar[j] + ba[c]), g = rec_sigmoid(ai[j] + bi[c]);
+        const float log_a = -rate[c] * r;
+        const size_t at = (size_t)t * width + c;
+        a_out[at] = expf(log_a);
+        b_out[at] = sqrtf(-expm1f(2.f * log_a)) * g * u[at];          // sqrt(1 - a^2) without the cancellation near a = 1
+    }
+}
+
+extern "C" int kva_block_gates(float *a_out, float *b_out, const float *u, int tokens, int width, int blocks, const void *wa,
+                               const void *wi, int w_dtype, const float *ba, const float *bi, const float *rate,
+                               hipStream_t stream) {
+    KVA_REQUIRE(a_out && b_out && u && wa && wi && ba && bi && rate, "block_gates: missing operand");
+    KVA_REQUIRE(tokens >= 0 && width > 0 && blocks > 0 && width % blocks == 0, "block_gates: %d channels in %d equal runs", width, blocks);
+    KVA_REQUIRE(w_dtype == KVA_BF16 || w_dtype == KVA_F32, "block_gates: unsupported dtype");
+    if (tokens == 0) return KVA_OK;
+    const int bs = width / blocks;
+    KVA_REQUIRE(blocks <= 65535 && (tokens + 15) / 16 <= 65535, "block_gates: too many runs or tokens for one launch");
+    hipLaunchKernelGGL(block_gates_kernel, dim3((bs + 63) / 64, blocks, (tokens + 15) / 16), dim3(256), 0, stream, a_out, b_out,
+                       u, tokens, width, bs, wa, wi, w_dtype, ba, bi, rate);
+    KVA_CHECK_LAUNCH("block_gates");
+    return KVA_OK;
+}
+
+// S_t = a_t S_(t-1) + b_t per channel over each entry's tokens in order, from the seat's S [width] (which takes
+// the last S_t); out[t, out_off + c] = S_t * act(gate[t, gate_off + c] + gate_bias[c]) * mul with act the tanh
+// form of gelu.  The recurrence is linear, so a workgroup of 16 segments x 16 channels cuts an entry's
+// tokens into 16 runs: every thread first folds its run into (A, B) with S_out = A S_in + B, the runs are
+// chained in order through LDS, and a second walk over the run writes the results.
+#define SCAN_SEGMENTS 16
+#define SCAN_CHANNELS 16
+__global__ void __launch_bounds__(256)
+linear_scan_gate_kernel(void *__restrict__ out, int out_dtype, int out_stride, int out_off, const float *__restrict__ a,
+                        const float *__restrict__ b, int width, const void *__restrict__ gate, int gate_dtype,
+                        int gate_stride, int gate_off, const float *__restrict__ gate_bias, float *__restrict__ state,
+                        size_t seat_stride, int state_off, const int *__restrict__ entry_q_start,
+                        const int *__restrict__ entry_seat, float mul) {
+    __shared__ float As[SCAN_SEGMENTS][SCAN_CHANNELS], Bs[SCAN_SEGMENTS][SCAN_CHANNELS];
+    const int e = blockIdx.y;
+    const int q0 = entry_q_start[e], n = entry_q_start[e + 1] - q0;
+    if (n <= 0) return;
+    const int cl = threadIdx.x % SCAN_CHANNELS, seg = threadIdx.x / SCAN_CHANNELS;
+    const int c = blockIdx.x * SCAN_CHANNELS + cl;
+    const bool on = c < width;
+    const int per = (n + SCAN_SEGMENTS - 1) / SCAN_SEGMENTS;
+    const int lo = min(n, seg * per), hi = min(n, lo + per);
+    float A = 1.f, B = 0.f;
+    if (on)
+        for (int i = lo; i < hi; ++i) {
+            const size_t at = (size_t)(q0 + i) * width + c;
+            const float av = a[at];
+            A *= av;
+            B = av * B + b[at];
+        }
+    As[seg][cl] = A;
+    Bs[seg][cl] = B;
+    __syncthreads();
+    if (!on) return;
+    float *st = state + (size_t)entry_seat[e] * seat_stride + state_off + c;
+    float S = *st;
+    for (int s2 = 0; s2 < seg; ++s2) S = As[s2][cl] * S + Bs[s2][cl];
+    const float gb = gate_bias ? gate_bias[c] : 0.f;
+    for (int i = lo; i < hi; ++i) {
+        const size_t at = (size_t)(q0 + i) * width + c;
+        S = a[at] * S + b[at];
+        const float g = rec_ld(gate, gate_dtype, (size_t)(q0 + i) * gate_stride + gate_off + c) + gb;
+        const float act = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+        rec_st(out, out_dtype, (size_t)(q0 + i) * out_stride + out_off + c, S * act * mul);
+    }
+    // the last segment's S is the entry's last state (an empty last segment holds it as its start)
+    if (seg == SCAN_SEGMENTS - 1) *st = S;
+}
+
+extern "C" int kva_linear_scan_gate(void *out, int out_dtype, int out_stride, int out_off, const float *a, const float *b,
+                                    int width, const void *gate, int gate_dtype, int gate_stride, int gate_off,
+                                    const float *gate_bias, float *state, long long seat_stride, int state_off,
+                                    const int *entry_q_start, const int *entry_seat, int entries, float mul,
+                                    hipStream_t stream) {
+    KVA_REQUIRE(out && a && b && gate && state && entry_q_start && entry_seat, "linear_scan_gate: missing operand");
+    KVA_REQUIRE(width > 0 && entries >= 0 && entries <= 65535, "linear_scan_gate: bad sizes");
+    if (entries == 0) return KVA_OK;
+    hipLaunchKernelGGL(linear_scan_gate_kernel, dim3((width + SCAN_CHANNELS - 1) / SCAN_CHANNELS, entries), dim3(256), 0, stream,
+                       out, out_dtype, out_stride, out_off, a, b, width, gate, gate_dtype, gate_stride, gate_off, gate_bias,
+                       state, (size_t)seat_stride, state_off, entry_q_start, entry_seat, mul);
+    KVA_CHECK_LAUNCH("linear_scan_gate");
+    return KVA_OK;
+}
+
+// ---- a matrix memory with exponential gates -----------------------------------------------------------
+// Per head a matrix S [dim, vdim], a vector n [dim] and a running maximum m (all zero at a request's start).
+// With the token's log input gate i = cap tanh(zi / cap), log forget gate f = logsigmoid(cap tanh(zf / cap)):
+//   m' = max(f + m, i);  S <- e^(f + m - m') S + e^(i - m') k v^T;  n <- e^(f + m - m') n + e^(i - m') k;
+//   o = S^T q / (max(|n . q|, e^(-m')) + 1e-6),  q times q_mul.
+// zi, zf come as fp32 rows [T, 2 heads] (input gates first).  One wavefront takes 16 value columns of a head:
+// lane = 16 r + c owns rows r, r + 4, ... of column c of S in LDS, and a copy of its rows of n; tokens are
+// staged 16 at a time.  The seat's state row holds S [heads, dim, vdim], then n and then m once per
+// wavefront, [heads, ceil(vdim / 16), dim] and [heads, ceil(vdim / 16)]: kva_matrix_memory_state says how much.
+#define MM_STAGE 16
+__global__ void __launch_bounds__(KVA_WAVE)
+matrix_memory_kernel(float *__restrict__ out, float *__restrict__ state, size_t seat_stride, int state_off,
+                     const void *__restrict__ y, int y_dtype, int y_stride, int q_off, int k_off, int v_off,
+                     const float *__restrict__ gates, float cap, float q_mul, const int *__restrict__ entry_q_start,
+                     const int *__restrict__ entry_seat, int heads, int dim, int vdim) {
+    extern __shared__ float lds[];
+    const int e = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * REC_COLS;
+    const int q0 = entry_q_start[e], n = entry_q_start[e + 1] - q0;
+    if (n <= 0) return;
+    const int lane = threadIdx.x, c = lane % REC_COLS, rg = lane / REC_COLS;
+    const int col = col0 + c;
+    const bool col_on = col < vdim;
+    float *S = lds;                                   // [dim][16]
+    float *N = S + (size_t)dim * REC_COLS;            // [dim][16]: every column's lanes keep their own copy
+    float *qs = N + (size_t)dim * REC_COLS;           // [MM_STAGE][dim]
+    float *ks = qs + (size_t)MM_STAGE * dim;          // [MM_STAGE][dim]
+    float *vs = ks + (size_t)MM_STAGE * dim;          // [MM_STAGE][16]
+    float *gs = vs + MM_STAGE * REC_COLS;             // [MM_STAGE][2]: log input gate, log forget gate
+    float *row = state + (size_t)entry_seat[e] * seat_stride + state_off;
+    float *S_g = row + (size_t)h * dim * vdim;
+    // (every wavefront reads and writes its own copy of n and m: no wavefront waits for another)
+    const int tiles = gridDim.x, tile = blockIdx.x;
+    float *n_g = row + (size_t)heads * dim * vdim + ((size_t)h * tiles + tile) * dim;
+    float *m_g = row + (size_t)heads * dim * vdim + (size_t)heads * tiles * dim + (size_t)h * tiles + tile;
+    for (int r = rg; r < dim; r += REC_ROWGROUPS) {
+        S[r * REC_COLS + c] = col_on ? S_g[(size_t)r * vdim + col] : 0.f;
+        N[r * REC_COLS + c] = n_g[r];
+    }
+    float m = *m_g;
+    for (int t0 = 0; t0 < n; t0 += MM_STAGE) {
+        const int cnt = min(MM_STAGE, n - t0);
+        __syncthreads();
+        for (int i = lane; i < cnt * dim; i += KVA_WAVE) {
+            const int tt = i / dim, r = i % dim;
+            const size_t at = (size_t)(q0 + t0 + tt) * y_stride;
+            qs[tt * dim + r] = rec_ld(y, y_dtype, at + q_off + h * dim + r) * q_mul;
+            ks[tt * dim + r] = rec_ld(y, y_dtype, at + k_off + h * dim + r);
+        }
+        for (int i = lane; i < cnt * REC_COLS; i += KVA_WAVE) {
+            const int tt = i / REC_COLS, cc = i % REC_COLS;
+            vs[i] = col0 + cc < vdim ? rec_ld(y, y_dtype, (size_t)(q0 + t0 + tt) * y_stride + v_off + h * vdim + col0 + cc) : 0.f;
+        }
+        if (lane < cnt) {
+            const float zi = gates[(size_t)(q0 + t0 + lane) * 2 * heads + h];
+            const float zf = gates[(size_t)(q0 + t0 + lane) * 2 * heads + heads + h];
+            const float f = cap * tanhf(zf / cap);
+            gs[2 * lane] = cap * tanhf(zi / cap);
+            gs[2 * lane + 1] = -rec_softplus(-f);         // logsigmoid
+        }
+        __syncthreads();
+        for (int tt = 0; tt < cnt; ++tt) {
+            const float gi = gs[2 * tt], gf = gs[2 * tt + 1];
+            const float m_new = fmaxf(gf + m, gi);
+            const float keep = expf(gf + m - m_new), take = expf(gi - m_new);
+            m = m_new;
+            const float tv = take * vs[tt * REC_COLS + c];
+            float num = 0.f, nq = 0.f;
+            for (int r = rg; r < dim; r += REC_ROWGROUPS) {
+                const float kv = ks[tt * dim + r], qv = qs[tt * dim + r];
+                const float sv = keep * S[r * REC_COLS + c] + kv * tv;
+                const float nv = keep * N[r * REC_COLS + c] + take * kv;
+                S[r * REC_COLS + c] = sv;
+                N[r * REC_COLS + c] = nv;
+                num += sv * qv;
+                nq += nv * qv;
+            }
+            num = rec_column_sum(num);
+            nq = rec_column_sum(nq);
+            const float den = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
+            if (rg == 0 && col_on) out[(size_t)(q0 + t0 + tt) * heads * vdim + (size_t)h * vdim + col] = num / den;
+        }
+    }
+    for (int r = rg; r < dim; r += REC_ROWGROUPS) {
+        if (col_on) S_g[(size_t)r * vdim + col] = S[r * REC_COLS + c];
+        if (c == 0) n_g[r] = N[r * REC_COLS + c];
+    }
+    if (lane == 0) *m_g = m;
+}
+
+extern "C" int kva_matrix_memory_state(int heads, int dim, int vdim) {
+    const int tiles = (vdim + REC_COLS - 1) / REC_COLS;
+    return heads * dim * vdim + heads * tiles * (dim + 1);
+}
+
+extern "C" int kva_matrix_memory(float *out, float *state, long long seat_stride, int state_off, const void *y, int y_dtype,
+                                 int y_stride, int q_off, int k_off, int v_off, const float *gates, float cap, float q_mul,
+                                 const int *entry_q_start, const int *entry_seat, int entries, int heads, int dim, int vdim,
+                                 hipStream_t stream) {
+    KVA_REQUIRE(out && state && y && gates && entry_q_start && entry_seat, "matrix_memory: missing operand");
+    KVA_REQUIRE(heads > 0 && dim > 0 && dim <= REC_MAX_DIM && vdim > 0 && cap > 0.f, "matrix_memory: bad sizes (key size up to %d)", REC_MAX_DIM);
+    KVA_REQUIRE(entries >= 0 && entries <= 65535 && heads <= 65535, "matrix_memory: bad batch");
+    if (entries == 0) return KVA_OK;
+    const size_t lds = ((size_t)2 * dim * REC_COLS + (size_t)2 * MM_STAGE * dim + MM_STAGE * REC_COLS + 2 * MM_STAGE) * sizeof(float);
+    KVA_REQUIRE(lds <= 160 * 1024, "matrix_memory: a key size of %d does not fit the local memory", dim);
+    if (lds > 64 * 1024)
+        hipFuncSetAttribute(reinterpret_cast<const void *>(matrix_memory_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(matrix_memory_kernel, dim3((vdim + REC_COLS - 1) / REC_COLS, heads, entries), dim3(KVA_WAVE), lds, stream,
+                       out, state, (size_t)seat_stride, state_off, y, y_dtype, y_stride, q_off, k_off, v_off, gates, cap, q_mul,
+                       entry_q_start, entry_seat, heads, dim, vdim);
+    KVA_CHECK_LAUNCH("matrix_memory");
     return KVA_OK;
 }

@@ -113,16 +113,17 @@ extern "C" int kva_stream_join(void *out, int out_dtype, void *x, int x_dtype, c
 }
 
 // out[t, i] = act(gu[t, i]) * gu[t, inter + i]
-__global__ void act_mul_kernel(void *__restrict__ out, const void *__restrict__ gu, int dtype, int inter, int act) {
+__global__ void act_mul_kernel(void *__restrict__ out, const void *__restrict__ gu, int dtype, int inter, int act,
+                               float limit) {
     const size_t t = blockIdx.y;
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= inter) return;
     const float g = ld_as_float(gu, dtype, t * 2 * inter + i), u = ld_as_float(gu, dtype, t * 2 * inter + inter + i);
-    st_from_float(out, dtype, t * inter + i, kva_activate(g, act) * u);
+    st_from_float(out, dtype, t * inter + i, kva_gated_activate(g, u, act, limit));
 }
 
 // bf16, inter a multiple of 8: a thread takes 8 neighbouring columns with 16-byte loads and stores
-__global__ void act_mul_vec_kernel(uint4 *__restrict__ out, const uint4 *__restrict__ gu, int inter8, int act) {
+__global__ void act_mul_vec_kernel(uint4 *__restrict__ out, const uint4 *__restrict__ gu, int inter8, int act, float limit) {
     const size_t t = blockIdx.y;
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= inter8) return;
@@ -133,24 +134,25 @@ __global__ void act_mul_vec_kernel(uint4 *__restrict__ out, const uint4 *__restr
     for (int j = 0; j < 4; ++j) {
         const float g0 = bf16_bits_to_float((uint16_t)(gw[j] & 0xffffu)), g1 = bf16_bits_to_float((uint16_t)(gw[j] >> 16));
         const float u0 = bf16_bits_to_float((uint16_t)(uw[j] & 0xffffu)), u1 = bf16_bits_to_float((uint16_t)(uw[j] >> 16));
-        ow[j] = (uint32_t)float_to_bf16_bits(kva_activate(g0, act) * u0) |
-                ((uint32_t)float_to_bf16_bits(kva_activate(g1, act) * u1) << 16);
+        ow[j] = (uint32_t)float_to_bf16_bits(kva_gated_activate(g0, u0, act, limit)) |
+                ((uint32_t)float_to_bf16_bits(kva_gated_activate(g1, u1, act, limit)) << 16);
     }
     out[t * inter8 + i] = make_uint4(ow[0], ow[1], ow[2], ow[3]);
 }
 
-extern "C" int kva_act_mul(void *out, const void *gate_up, int rows, int inter, int act, int dtype, hipStream_t stream) {
+extern "C" int kva_act_mul(void *out, const void *gate_up, int rows, int inter, int act, float limit, int dtype,
+                           hipStream_t stream) {
     KVA_REQUIRE(rows >= 0 && rows <= 65535 && inter > 0, "act_mul: bad sizes");
-    KVA_REQUIRE(act >= KVA_ACT_SILU && act <= KVA_ACT_GELU_TANH, "act_mul: unknown activation %d", act);
+    KVA_REQUIRE(act >= KVA_ACT_SILU && act <= KVA_ACT_SWISH_CLAMPED, "act_mul: unknown activation %d", act);
     if (rows == 0) return KVA_OK;
     if (dtype == KVA_BF16 && inter % 8 == 0) {
         hipLaunchKernelGGL(act_mul_vec_kernel, dim3((inter / 8 + 255) / 256, rows), dim3(256), 0, stream, (uint4 *)out,
-                           (const uint4 *)gate_up, inter / 8, act);
+                           (const uint4 *)gate_up, inter / 8, act, limit);
         KVA_CHECK_LAUNCH("act_mul");
         return KVA_OK;
     }
     hipLaunchKernelGGL(act_mul_kernel, dim3((inter + 255) / 256, rows), dim3(256), 0, stream, out, gate_up, dtype,
-                       inter, act);
+                       inter, act, limit);
     KVA_CHECK_LAUNCH("act_mul");
     return KVA_OK;
 }
@@ -330,5 +332,149 @@ extern "C" int kva_table_gate(void *out, const void *z, int dtype, const void *t
     hipLaunchKernelGGL(table_gate_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, out, z, dtype, table,
                        table_dtype, table_width, table_rows, col0, ids, feedback, dim, act, rows);
     KVA_CHECK_LAUNCH("table_gate");
+    return KVA_OK;
+}
+
+// ---- an activation over rows, with a bias ---------------------------------------------------------
+// out[t, i] = act(x[t, i] + bias[i]) (the bias is optional): the middle of a feed-forward that is not gated.
+__global__ void bias_act_kernel(void *__restrict__ out, const void *__restrict__ x, int dtype, const float *__restrict__ bias,
+                                int width, int act, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float z = ld_as_float(x, dtype, i) + (bias ? bias[i % width] : 0.f);
+    st_from_float(out, dtype, i, kva_activate(z, act));
+}
+
+extern "C" int kva_bias_act(void *out, const void *x, int dtype, const float *bias, int rows, int width, int act,
+                            hipStream_t stream) {
+    KVA_REQUIRE(out && x && rows >= 0 && width > 0, "bias_act: missing operand or bad sizes");
+    KVA_REQUIRE(act >= KVA_ACT_SILU && act <= KVA_ACT_GELU_TANH, "bias_act: unknown activation %d", act);
+    if (rows == 0) return KVA_OK;
+    const size_t n = (size_t)rows * width;
+    hipLaunchKernelGGL(bias_act_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, out, x, dtype, bias, width,
+                       act, n);
+    KVA_CHECK_LAUNCH("bias_act");
+    return KVA_OK;
+}
+
+// ---- several copies of the stream (hyper-connections) -----------------------------------------------
+// The residual stream is S copies x_1 .. x_S of every row, kept side by side: x [rows, S, width] fp32.
+// One launch does what lies between two branches, a workgroup a row:
+//   (1) with y, the branch output that is still to enter: all copies at once from the old ones,
+//       x_t <- sum_s mix[s, t] x_s + mult * out_w[t] * y;
+//   (2) with out: u = sum_s in_w[s] x_s of the new copies, then the layer norm with weight and bias,
+//       out = (u - mean) / sqrt(var + eps) * w + b.
+// With row_idx only the named rows are read (and nothing is written back): the model's last norm.
+// S = 1 with mix = out_w = in_w = 1 is a plain residual stream whose branches enter times `mult`.
+#define HYPER_MAX_STREAMS 8
+
+struct HyperCoefficients {
+    float mix[HYPER_MAX_STREAMS * HYPER_MAX_STREAMS], out_w[HYPER_MAX_STREAMS], in_w[HYPER_MAX_STREAMS];
+};
+
+template <int S>
+__global__ void __launch_bounds__(256)
+hyper_step_kernel(float *__restrict__ x, const void *__restrict__ y, int y_dtype, const float *__restrict__ mix,
+                  const float *__restrict__ out_w, float mult, const float *__restrict__ in_w,
+                  const void *__restrict__ nw, const void *__restrict__ nb, int w_dtype, float eps,
+                  void *__restrict__ out, int out_dtype, const int *__restrict__ row_idx, int width) {
+    extern __shared__ float row_s[];
+    __shared__ float red_s[4];
+    __shared__ HyperCoefficients co;
+    const int r = blockIdx.x;
+    const size_t row = (size_t)(row_idx ? row_idx[r] : r);
+    if (threadIdx.x < S * S) co.mix[threadIdx.x] = y ? mix[threadIdx.x] : 0.f;
+    if (threadIdx.x < S) {
+        co.out_w[threadIdx.x] = y ? out_w[threadIdx.x] * mult : 0.f;
+        co.in_w[threadIdx.x] = out ? in_w[threadIdx.x] : 0.f;
+    }
+    __syncthreads();
+    float *xr = x + row * S * width;
+    float sum = 0.f;
+    for (int j = threadIdx.x; j < width; j += blockDim.x) {
+        float v[S];
+#pragma unroll
+        for (int s = 0; s < S; ++s) v[s] = xr[(size_t)s * width + j];
+        if (y) {
+            const float yv = ld_as_float(y, y_dtype, row * width + j);
+            float nv[S];
+#pragma unroll
+            for (int t = 0; t < S; ++t) {
+                float acc = 0.f;
+#pragma unroll
+                for (int s = 0; s < S; ++s) acc += co.mix[s * S + t] * v[s];
+                nv[t] = acc + co.out_w[t] * yv;
+            }
+#pragma unroll
+            for (int t = 0; t < S; ++t) {
+                v[t] = nv[t];
+                if (!row_idx) xr[(size_t)t * width + j] = nv[t];
+            }
+        }
+        if (out) {
+            float u = 0.f;
+#pragma unroll
+            for (int s = 0; s < S; ++s) u += co.in_w[s] * v[s];
+            row_s[j] = u;
+            sum += u;
+        }
+    }
+    if (!out) return;
+    const float mean = block_sum(sum, red_s, blockDim.x / KVA_WAVE) / (float)width;
+    float sq = 0.f;
+    for (int j = threadIdx.x; j < width; j += blockDim.x) {
+        const float d = row_s[j] - mean;
+        sq += d * d;
+    }
+    const float inv = 1.0f / sqrtf(block_sum(sq, red_s, blockDim.x / KVA_WAVE) / (float)width + eps);
+    for (int j = threadIdx.x; j < width; j += blockDim.x)
+        st_from_float(out, out_dtype, (size_t)r * width + j,
+                      (row_s[j] - mean) * inv * ld_as_float(nw, w_dtype, j) + (nb ? ld_as_float(nb, w_dtype, j) : 0.f));
+}
+
+extern "C" int kva_hyper_step(float *x, int streams, const void *y, int y_dtype, const float *mix, const float *out_w,
+                              float mult, const float *in_w, const void *norm_w, const void *norm_b, int w_dtype, float eps,
+                              void *out, int out_dtype, const int *row_idx, int rows, int width, hipStream_t stream) {
+    KVA_REQUIRE(x && rows >= 0 && width > 0 && width <= 16000, "hyper_step: width %d must lie in 1..16000", width);
+    KVA_REQUIRE(streams >= 1 && streams <= HYPER_MAX_STREAMS, "hyper_step: %d copies of the stream (1..%d are built)", streams,
+                HYPER_MAX_STREAMS);
+    KVA_REQUIRE(!y || (mix && out_w), "hyper_step: a branch output enters through a mixing matrix and output weights");
+    KVA_REQUIRE(!out || (in_w && norm_w && eps >= 0.f), "hyper_step: the read-out needs input weights and a norm");
+    KVA_REQUIRE(y || out, "hyper_step: nothing to do");
+    KVA_REQUIRE(!row_idx || out, "hyper_step: rows are gathered for the read-out only");
+    if (rows == 0) return KVA_OK;
+    const size_t lds = (size_t)width * sizeof(float);
+#define KVA_HYPER_CASE(S)                                                                                               \
+    case S:                                                                                                             \
+        hipLaunchKernelGGL(hyper_step_kernel<S>, dim3(rows), dim3(256), lds, stream, x, y, y_dtype, mix, out_w, mult, in_w,  \
+                           norm_w, norm_b, w_dtype, eps, out, out_dtype, row_idx, width);                              \
+        break;
+    switch (streams) {
+        KVA_HYPER_CASE(1) KVA_HYPER_CASE(2) KVA_HYPER_CASE(3) KVA_HYPER_CASE(4)
+        KVA_HYPER_CASE(5) KVA_HYPER_CASE(6) KVA_HYPER_CASE(7) KVA_HYPER_CASE(8)
+    }
+#undef KVA_HYPER_CASE
+    KVA_CHECK_LAUNCH("hyper_step");
+    return KVA_OK;
+}
+
+// every row of `first` [rows, width] (any storage type) into all S copies of x [rows, S, width] fp32: the
+// stream as the embedding leaves it
+__global__ void hyper_fill_kernel(float *__restrict__ x, const void *__restrict__ first, int dtype, int streams, int width,
+                                  size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const size_t t = i / width, j = i % width;
+    const float v = ld_as_float(first, dtype, i);
+    for (int s = 0; s < streams; ++s) x[(t * streams + s) * width + j] = v;
+}
+
+extern "C" int kva_hyper_fill(float *x, const void *first, int dtype, int streams, int rows, int width, hipStream_t stream) {
+    KVA_REQUIRE(x && first && streams >= 1 && rows >= 0 && width > 0, "hyper_fill: missing operand or bad sizes");
+    if (rows == 0) return KVA_OK;
+    const size_t n = (size_t)rows * width;
+    hipLaunchKernelGGL(hyper_fill_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, first, dtype, streams,
+                       width, n);
+    KVA_CHECK_LAUNCH("hyper_fill");
     return KVA_OK;
 }

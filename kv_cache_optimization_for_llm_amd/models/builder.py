@@ -11,6 +11,7 @@ from . import llama as _llama   # noqa: F401  (registers LlamaForCausalLM)
 from . import gadopel as _gadopel   # noqa: F401  (registers Gadopel)
 from . import radilix as _radilix   # noqa: F401  (registers Radilix)
 from . import lomodra as _lomodra   # noqa: F401  (registers Lomodra)
+from . import bonusun as _bonusun   # noqa: F401  (registers Bonusun)
 from ..config.registry import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, STREAM_OPS, architecture_for)
 from ..models.spec import LayerCall, ModelSpec, TensorSpec
 from ..ops import kernels as K
@@ -92,6 +93,8 @@ class Model:
         self.stream_dtype = {None: dtype, "float32": torch.float32, "bfloat16": torch.bfloat16}[spec.residual_dtype]
         if self.stream_dtype == torch.bfloat16 and dtype == torch.float32:
             self.stream_dtype = dtype
+        if int(spec.streams) < 1 or (int(spec.streams) > 1 and self.stream_dtype != torch.float32):
+            raise ValueError("several copies of the stream are kept in 32-bit (residual_dtype='float32')")
         self.calls = resolve_order(spec)
         self.embedding: Optional[torch.Tensor] = None
         self.head: Optional[Linear] = None
@@ -144,7 +147,7 @@ class Model:
         widest = max((sum(part.activation_elements() for part in b.parts()) for b in self.blocks), default=0)
         widest += max((op.activation_elements() for op in self.stream_ops), default=0)
         rows = int(tokens if logit_rows is None else logit_rows)
-        return int(tokens) * (3 * self.spec.hidden_size + 2 * widest) * elem + rows * 4 * self.spec.vocab_size
+        return int(tokens) * ((2 + int(self.spec.streams)) * self.spec.hidden_size + 2 * widest) * elem + rows * 4 * self.spec.vocab_size
 
     def graph_safe(self) -> bool:
         """Whether every part may be captured into a HIP graph."""
@@ -229,14 +232,15 @@ class Model:
         """Runs the batch's tokens through every layer call and returns fp32 logits
         ``[len(batch.logit_rows), vocab]``."""
         T = batch.num_tokens
-        hidden = torch.empty((T, self.spec.hidden_size), dtype=self.stream_dtype, device=self.device)
+        S = int(self.spec.streams)
+        hidden = torch.empty((T, S * self.spec.hidden_size), dtype=self.stream_dtype, device=self.device)
         delta = None
         first = None            # the embedding output in the compute type, for operations that read it again
         first_norm = self.blocks[self.calls[0][0].layer].first_norm() if self.calls else self.final_norm
         prep = first_norm.prepared_by_product() if first_norm is not None else None
         if (T <= self.GATHER_PREP_MAX_ROWS and prep is not None and prep[1] == self.spec.hidden_size
                 and self.dtype == torch.bfloat16 and self.embedding.dtype == torch.bfloat16
-                and self.stream_dtype == torch.bfloat16 and not self.stream_ops
+                and self.stream_dtype == torch.bfloat16 and not self.stream_ops and S == 1
                 and self.spec.hidden_size % 8 == 0 and self.spec.embedding_scale == 1.0):
             # a few tokens: the gather prepares the first norm as a product's epilogue would, and
             # the first product finishes it (or one kernel does, as the norm kernel would have)
@@ -245,6 +249,15 @@ class Model:
             K.embed_gather_prep(self.embedding, batch.token_ids, hidden, scaled, sumsq, prep[0],
                                 getattr(batch, "feedback", None))
             delta = NormedRows(scaled, sumsq, prep[1], prep[2], first_norm)
+        elif S > 1:
+            # several copies of the stream: every copy starts as the embedding output
+            if self.stream_ops:
+                raise TypeError("operations between layers take a stream of one copy")
+            one = torch.empty((T, self.spec.hidden_size), dtype=self.stream_dtype, device=self.device)
+            K.embed_gather(self.embedding, batch.token_ids, one, getattr(batch, "feedback", None))
+            if self.spec.embedding_scale != 1.0:
+                K.scale_softcap(one, self.spec.embedding_scale)
+            K.hyper_fill(hidden, one, S)
         else:
             K.embed_gather(self.embedding, batch.token_ids, hidden, getattr(batch, "feedback", None))
             if self.spec.embedding_scale != 1.0:

@@ -18,7 +18,7 @@ class TensorSpec:
     """One tensor a part reads from the checkpoint.
 
     ``init`` names the random-weights rule: ``"normal"`` (N(0, 0.02)), ``"norm"``
-    (1 + U(-0.1, 0.1)) or ``"zeros"``.  ``role`` is ``"matrix"`` (takes the engine's compute
+    (1 + U(-0.1, 0.1)), ``"eye"`` (a square matrix: the identity + U(-0.1, 0.1)) or ``"zeros"``.  ``role`` is ``"matrix"`` (takes the engine's compute
     dtype unless stored in 32-bit), ``"vector"`` (same rule) or ``"table"`` (integers, int32).
     """
 
@@ -83,6 +83,9 @@ class ModelSpec:
     # Type the residual stream is kept in: None = the engine's compute type; "float32" keeps the
     # stream (and its sums) in 32-bit also where products and activations are bfloat16.
     residual_dtype: Optional[str] = None
+    # Copies of the stream kept side by side per row (hyper-connections): the stream is [T, streams * hidden],
+    # every copy starts as the embedding output, and the blocks and the final norm know what to do with them.
+    streams: int = 1
     ignorable_tensors: Tuple[str, ...] = ()   # fnmatch patterns of tensors that may be present unused
 
 

@@ -583,6 +583,9 @@ def norm_into_stream(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps
 
 
 ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2}
+# gated forms only: act(gate) * up with "swish_clamped" = g sigmoid(1.702 g) (u + 1), g = min(gate, limit),
+# u = clamp(up, -limit, limit)
+GATED_ACTIVATIONS = dict(ACTIVATIONS, swish_clamped=3)
 
 
 def table_gate(z: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, col0: int, out: torch.Tensor, activation: str,
@@ -603,17 +606,76 @@ def table_gate(z: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, col0: in
     return out
 
 
-def act_mul(gate_up: torch.Tensor, out: torch.Tensor, activation: str) -> torch.Tensor:
+def act_mul(gate_up: torch.Tensor, out: torch.Tensor, activation: str, limit: float = 0.0) -> torch.Tensor:
     """out[t, i] = act(gate_up[t, i]) * gate_up[t, I + i] with ``activation`` one of silu, relu,
-    gelu_tanh (0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))))."""
+    gelu_tanh (0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))), or the gated form swish_clamped
+    with its ``limit``."""
     rows, inter = out.shape
-    if activation not in ACTIVATIONS:
-        raise KernelError(f"act_mul: activation {activation!r} is not one of {sorted(ACTIVATIONS)}")
+    if activation not in GATED_ACTIVATIONS:
+        raise KernelError(f"act_mul: activation {activation!r} is not one of {sorted(GATED_ACTIVATIONS)}")
     if gate_up.shape != (rows, 2 * inter) or gate_up.dtype != out.dtype:
         raise KernelError(f"act_mul: gate_up {tuple(gate_up.shape)} does not fit out {tuple(out.shape)}")
-    check(hip_lib().kva_act_mul(_dev(out, "out"), _dev(gate_up, "gate_up"), rows, inter, ACTIVATIONS[activation],
-                                dtype_code(out.dtype), _stream()), "act_mul")
+    check(hip_lib().kva_act_mul(_dev(out, "out"), _dev(gate_up, "gate_up"), rows, inter, GATED_ACTIVATIONS[activation],
+                                float(limit), dtype_code(out.dtype), _stream()), "act_mul")
     return out
+
+
+def bias_act(x: torch.Tensor, out: torch.Tensor, activation: str, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out = act(x + bias)`` element by element (``bias`` fp32, one value per column, optional); ``out``
+    may be ``x``."""
+    if activation not in ACTIVATIONS:
+        raise KernelError(f"bias_act: activation {activation!r} is not one of {sorted(ACTIVATIONS)}")
+    if x.dim() != 2 or out.shape != x.shape or out.dtype != x.dtype \
+            or (bias is not None and (bias.shape != (x.shape[1],) or bias.dtype != torch.float32)):
+        raise KernelError(f"bias_act: x {tuple(x.shape)} and out {tuple(out.shape)} do not fit")
+    check(hip_lib().kva_bias_act(_dev(out, "out"), _dev(x, "x"), dtype_code(x.dtype), _opt(bias, "bias"), x.shape[0],
+                                 x.shape[1], ACTIVATIONS[activation], _stream()), "bias_act")
+    return out
+
+
+def hyper_step(x: torch.Tensor, streams: int, *, y: Optional[torch.Tensor] = None, mix: Optional[torch.Tensor] = None,
+               out_w: Optional[torch.Tensor] = None, mult: float = 1.0, in_w: Optional[torch.Tensor] = None,
+               norm_weight: Optional[torch.Tensor] = None, norm_bias: Optional[torch.Tensor] = None, eps: float = 0.0,
+               out: Optional[torch.Tensor] = None, row_idx: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """One step between two branches over ``streams`` copies of the residual stream, ``x`` fp32 ``[T, streams *
+    width]`` (a row's copies side by side).  With ``y`` ``[T, width]`` every copy is replaced, all at once from
+    the old ones: ``x_t <- sum_s mix[s, t] x_s + mult * out_w[t] * y``.  With ``out`` the new copies are read out,
+    ``u = sum_s in_w[s] x_s``, and normed: ``out = (u - mean) / sqrt(var + eps) * norm_weight + norm_bias``.
+    ``row_idx``: only these rows are read out, and nothing is written back.  ``mix`` ``[streams, streams]``,
+    ``out_w`` and ``in_w`` ``[streams]`` are fp32."""
+    S = int(streams)
+    if x.dim() != 2 or x.dtype != torch.float32 or x.shape[1] % S:
+        raise KernelError(f"hyper_step: x {tuple(x.shape)} is not fp32 [T, {S} copies * width]")
+    T, width = x.shape[0], x.shape[1] // S
+    if y is not None and (y.shape != (T, width) or mix is None or out_w is None or mix.shape != (S, S)
+                          or out_w.shape != (S,) or mix.dtype != torch.float32 or out_w.dtype != torch.float32):
+        raise KernelError("hyper_step: a branch output [T, width] enters through fp32 mix [S, S] and out_w [S]")
+    rows = T
+    if out is not None:
+        rows = T if row_idx is None else row_idx.shape[0]
+        if out.shape != (rows, width) or in_w is None or in_w.shape != (S,) or in_w.dtype != torch.float32 \
+                or norm_weight is None or norm_weight.shape != (width,) \
+                or (norm_bias is not None and (norm_bias.shape != (width,) or norm_bias.dtype != norm_weight.dtype)):
+            raise KernelError("hyper_step: the read-out needs out [rows, width], fp32 in_w [S] and a norm weight (and bias) [width]")
+    elif row_idx is not None:
+        raise KernelError("hyper_step: rows are gathered for the read-out only")
+    check(hip_lib().kva_hyper_step(
+        _dev(x, "x"), S, _opt(y, "y"), dtype_code(y.dtype) if y is not None else 0, _opt(mix, "mix"), _opt(out_w, "out_w"),
+        float(mult), _opt(in_w, "in_w"), _opt(norm_weight, "norm_weight"), _opt(norm_bias, "norm_bias"),
+        dtype_code(norm_weight.dtype) if norm_weight is not None else 0, float(eps), _opt(out, "out"),
+        dtype_code(out.dtype) if out is not None else 0, _opt(row_idx, "row_idx", torch.int32), rows, width, _stream()),
+        "hyper_step")
+    return out
+
+
+def hyper_fill(x: torch.Tensor, first: torch.Tensor, streams: int) -> torch.Tensor:
+    """Every row of ``first`` ``[T, width]`` into all ``streams`` copies of ``x`` fp32 ``[T, streams * width]``."""
+    T, width = first.shape
+    if x.shape != (T, int(streams) * width) or x.dtype != torch.float32:
+        raise KernelError(f"hyper_fill: x {tuple(x.shape)} does not hold {streams} copies of {tuple(first.shape)}")
+    check(hip_lib().kva_hyper_fill(_dev(x, "x"), _dev(first, "first"), dtype_code(first.dtype), int(streams), T, width,
+                                   _stream()), "hyper_fill")
+    return x
 
 
 def head_gate(x: torch.Tensor, gates: torch.Tensor, heads: int) -> torch.Tensor:
@@ -633,7 +695,8 @@ def qk_encode_cache(qkv: torch.Tensor, positions: torch.Tensor, num_q_heads: int
                     value_dim: int, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], interleaved: bool,
                     unit_eps: Optional[float], k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
                     slot_mapping: Optional[torch.Tensor], bias: Optional[torch.Tensor] = None,
-                    q_weight: Optional[torch.Tensor] = None, k_weight: Optional[torch.Tensor] = None) -> None:
+                    q_weight: Optional[torch.Tensor] = None, k_weight: Optional[torch.Tensor] = None,
+                    norm_first: bool = False) -> None:
     """Rotates the first ``2 * cos.shape[1]`` elements of every Q and K head of ``qkv``
     ``[T, nq d + nkv d + nkv value_dim]`` (pair i = elements (2i, 2i + 1) when ``interleaved``, else
     (i, i + rot / 2)), then - with ``unit_eps`` - divides every head by its root mean square; Q in
@@ -642,6 +705,8 @@ def qk_encode_cache(qkv: torch.Tensor, positions: torch.Tensor, num_q_heads: int
     column) is added to Q, K and V first: the projection's bias, applied here.  ``q_weight`` /
     ``k_weight`` (fp32 ``[head_dim]``, with ``unit_eps``): every query / key head is multiplied by it
     after the division - an RMS norm of the head with a weight shared by the heads.
+    ``norm_first``: the division and the weights come before the rotation instead (the normed head is
+    what is rotated).
     ``num_kv_heads = 0``: ``qkv`` holds queries alone (a layer that reads another layer's keys and
     values); nothing is written to a cache."""
     tokens = qkv.shape[0]
@@ -676,7 +741,7 @@ def qk_encode_cache(qkv: torch.Tensor, positions: torch.Tensor, num_q_heads: int
         _opt(slot_mapping if write else None, "slot_mapping", torch.int32), tokens, num_q_heads, num_kv_heads,
         head_dim, value_dim, rot, 1 if interleaved else 0, -1.0 if unit_eps is None else float(unit_eps),
         page_size, dtype_code(qkv.dtype), _opt(bias, "bias"), _opt(q_weight, "q_weight"), _opt(k_weight, "k_weight"),
-        _stream()), "qk_encode_cache")
+        1 if norm_first else 0, _stream()), "qk_encode_cache")
 
 
 def latent_encode_cache(y: torch.Tensor, kv_off: int, q_lat: torch.Tensor, cache: Optional[torch.Tensor],
@@ -1423,13 +1488,21 @@ def _state_row(state: torch.Tensor, offset: int, elements: int, what: str) -> in
 
 
 def causal_conv_act(y: torch.Tensor, col_off: int, weight: torch.Tensor, out: torch.Tensor, state: torch.Tensor,
-                    state_off: int, entry_q_start: torch.Tensor, entry_seat: torch.Tensor, max_q_len: int) -> torch.Tensor:
+                    state_off: int, entry_q_start: torch.Tensor, entry_seat: torch.Tensor, max_q_len: int,
+                    in_bias: Optional[torch.Tensor] = None, out_bias: Optional[torch.Tensor] = None,
+                    activation: Optional[str] = "silu") -> torch.Tensor:
     """A short causal convolution over time per channel, then silu: ``out[t, c] = silu(sum_j
     weight[c, j] * in[t - taps + 1 + j, c])`` with ``in`` the columns ``col_off ..`` of ``y``; the inputs
     before an entry's first token come from the seat's state (``taps - 1`` values per channel at
     ``state_off``, oldest first; zero for a fresh seat), which afterwards holds the entry's last ones.
-    ``out`` is fp32 ``[T, channels]``."""
+    ``out`` is fp32 ``[T, channels]``.  ``in_bias`` (fp32 per channel) is added to every input (the state
+    holds inputs with it), ``out_bias`` to every sum; ``activation`` is ``"silu"`` or ``None``."""
     tokens, channels = out.shape
+    for bias in (in_bias, out_bias):
+        if bias is not None and (bias.shape != (channels,) or bias.dtype != torch.float32):
+            raise KernelError("causal_conv_act: a bias is fp32, one value per channel")
+    if activation not in (None, "silu"):
+        raise KernelError(f"causal_conv_act: activation {activation!r} is neither None nor 'silu'")
     if weight.dim() != 2 or weight.shape[0] != channels or out.dtype != torch.float32 or y.dim() != 2 \
             or y.shape[0] != tokens or col_off < 0 or col_off + channels > y.shape[1]:
         raise KernelError(f"causal_conv_act: y {tuple(y.shape)}, weight {tuple(weight.shape)}, out {tuple(out.shape)} do not fit")
@@ -1439,7 +1512,8 @@ def causal_conv_act(y: torch.Tensor, col_off: int, weight: torch.Tensor, out: to
     check(hip_lib().kva_causal_conv_act(
         _dev(out, "out"), channels, _dev(y, "y"), dtype_code(y.dtype), y.shape[1], int(col_off), _dev(weight, "weight"),
         dtype_code(weight.dtype), _dev(state, "state"), seat_stride, int(state_off), qs, seat, entries, int(max_q_len),
-        channels, taps, _stream()), "causal_conv_act")
+        channels, taps, _opt(in_bias, "in_bias"), _opt(out_bias, "out_bias"), 1 if activation == "silu" else 0,
+        _stream()), "causal_conv_act")
     return out
 
 
@@ -1516,50 +1590,135 @@ def gated_linear_attention(y: torch.Tensor, q_off: int, k_off: int, v_off: int, 
     return out
 
 
+def block_gates(u: torch.Tensor, w_a: torch.Tensor, w_i: torch.Tensor, bias_a: torch.Tensor, bias_i: torch.Tensor,
+                rate: torch.Tensor, a_out: torch.Tensor, b_out: torch.Tensor) -> None:
+    """The decays and inputs of a real-gated linear recurrent unit for all tokens: with the channels of ``u``
+    fp32 ``[T, width]`` in ``blocks`` equal runs and the square matrices ``w_a``, ``w_i`` ``[blocks, bs, bs]``
+    (``[out, in]``, bf16 or fp32) of every run, ``r = sigmoid(w_a u_b + bias_a)``, ``i = sigmoid(w_i u_b + bias_i)``,
+    ``a_out = exp(-rate r)`` and ``b_out = sqrt(1 - a^2) i u``; everything fp32."""
+    T, width = u.shape
+    if w_a.dim() != 3 or w_a.shape != w_i.shape or w_a.shape[1] != w_a.shape[2] or w_a.shape[0] * w_a.shape[1] != width \
+            or w_a.dtype != w_i.dtype:
+        raise KernelError(f"block_gates: matrices {tuple(w_a.shape)} / {tuple(w_i.shape)} do not cut {width} channels into equal runs")
+    for t in (u, bias_a, bias_i, rate, a_out, b_out):
+        if t.dtype != torch.float32:
+            raise KernelError("block_gates: inputs, biases, rates and results are fp32")
+    if bias_a.numel() != width or bias_i.numel() != width or rate.shape != (width,) or a_out.shape != u.shape or b_out.shape != u.shape:
+        raise KernelError("block_gates: one bias and one rate per channel, results of u's shape")
+    check(hip_lib().kva_block_gates(_dev(a_out, "a_out"), _dev(b_out, "b_out"), _dev(u, "u"), T, width, w_a.shape[0],
+                                    _dev(w_a, "w_a"), _dev(w_i, "w_i"), dtype_code(w_a.dtype), _dev(bias_a, "bias_a"),
+                                    _dev(bias_i, "bias_i"), _dev(rate, "rate"), _stream()), "block_gates")
+
+
+def linear_scan_gate(a: torch.Tensor, b: torch.Tensor, gate: torch.Tensor, gate_off: int, gate_bias: Optional[torch.Tensor],
+                     out: torch.Tensor, out_off: int, state: torch.Tensor, state_off: int, entry_q_start: torch.Tensor,
+                     entry_seat: torch.Tensor, mul: float = 1.0) -> torch.Tensor:
+    """``S_t = a_t S_(t-1) + b_t`` per channel over every entry's tokens in order, from the seat's ``S`` fp32
+    ``[width]`` at ``state_off`` (which takes the last one); ``out[t, out_off + c] = S_t * gelu_tanh(gate[t,
+    gate_off + c] + gate_bias[c]) * mul``.  ``a``, ``b`` fp32 ``[T, width]``; ``gate`` and ``out`` may be wider."""
+    T, width = a.shape
+    if b.shape != a.shape or a.dtype != torch.float32 or b.dtype != torch.float32 or gate.dim() != 2 or gate.shape[0] != T \
+            or out.dim() != 2 or out.shape[0] != T or not 0 <= gate_off <= gate.shape[1] - width \
+            or not 0 <= out_off <= out.shape[1] - width:
+        raise KernelError(f"linear_scan_gate: a {tuple(a.shape)}, gate {tuple(gate.shape)}, out {tuple(out.shape)} do not fit")
+    if gate_bias is not None and (gate_bias.shape != (width,) or gate_bias.dtype != torch.float32):
+        raise KernelError("linear_scan_gate: the gate's bias is fp32, one value per channel")
+    seat_stride = _state_row(state, state_off, width, "linear_scan_gate")
+    qs, seat, entries = _entries((entry_q_start, entry_seat), "linear_scan_gate")
+    check(hip_lib().kva_linear_scan_gate(
+        _dev(out, "out"), dtype_code(out.dtype), out.shape[1], int(out_off), _dev(a, "a"), _dev(b, "b"), width,
+        _dev(gate, "gate"), dtype_code(gate.dtype), gate.shape[1], int(gate_off), _opt(gate_bias, "gate_bias"),
+        _dev(state, "state"), seat_stride, int(state_off), qs, seat, entries, float(mul), _stream()), "linear_scan_gate")
+    return out
+
+
+def matrix_memory_state(heads: int, dim: int, vdim: int) -> int:
+    """fp32 values of state :func:`matrix_memory` keeps per request."""
+    return int(hip_lib().kva_matrix_memory_state(int(heads), int(dim), int(vdim)))
+
+
+def matrix_memory(y: torch.Tensor, q_off: int, k_off: int, v_off: int, gates: torch.Tensor, cap: float, q_mul: float,
+                  out: torch.Tensor, state: torch.Tensor, state_off: int, entry_q_start: torch.Tensor,
+                  entry_seat: torch.Tensor, heads: int, dim: int, vdim: int) -> torch.Tensor:
+    """A matrix memory with exponential gates per head: with ``i = cap tanh(zi / cap)``, ``f = logsigmoid(cap
+    tanh(zf / cap))`` from ``gates`` fp32 ``[T, 2 heads]`` (``zi`` of all heads, then ``zf``) and a running maximum
+    ``m' = max(f + m, i)``: ``S <- e^(f + m - m') S + e^(i - m') k v^T``, ``n`` likewise with ``k`` alone, ``o =
+    S^T q / (max(|n . q|, e^(-m')) + 1e-6)`` with ``q`` times ``q_mul``.  q, k (``heads x dim``) and v (``heads x
+    vdim``) are columns of ``y``; ``out`` is fp32 ``[T, heads * vdim]``; S, n and m live in the seat's state row."""
+    T = out.shape[0]
+    if out.shape != (T, heads * vdim) or out.dtype != torch.float32 or y.dim() != 2 or y.shape[0] != T \
+            or gates.shape != (T, 2 * heads) or gates.dtype != torch.float32:
+        raise KernelError(f"matrix_memory: y {tuple(y.shape)}, gates {tuple(gates.shape)}, out {tuple(out.shape)} do not fit")
+    for off, n in ((q_off, heads * dim), (k_off, heads * dim), (v_off, heads * vdim)):
+        if not 0 <= off <= y.shape[1] - n:
+            raise KernelError("matrix_memory: q, k or v lies outside the projection's columns")
+    seat_stride = _state_row(state, state_off, matrix_memory_state(heads, dim, vdim), "matrix_memory")
+    qs, seat, entries = _entries((entry_q_start, entry_seat), "matrix_memory")
+    check(hip_lib().kva_matrix_memory(
+        _dev(out, "out"), _dev(state, "state"), seat_stride, int(state_off), _dev(y, "y"), dtype_code(y.dtype), y.shape[1],
+        int(q_off), int(k_off), int(v_off), _dev(gates, "gates"), float(cap), float(q_mul), qs, seat, entries, int(heads),
+        int(dim), int(vdim), _stream()), "matrix_memory")
+    return out
+
+
 HEAD_GATES = {"silu": 0, "sigmoid": 1}
 
 
-def head_norm_gate(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, gate: torch.Tensor, gate_off: int,
-                   out: torch.Tensor, out_off: int, heads: int, vdim: int, activation: str, mul: float = 1.0) -> torch.Tensor:
+def head_norm_gate(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, gate: Optional[torch.Tensor], gate_off: int,
+                   out: torch.Tensor, out_off: int, heads: int, vdim: int, activation: Optional[str], mul: float = 1.0) -> torch.Tensor:
     """``out[t, out_off + h vdim + j] = n(x)[t, h, j] * act(gate[t, gate_off + h vdim + j]) * mul`` where
     ``n`` divides every head by its root mean square (``sqrt(mean_j x^2 + eps)``) and multiplies by
-    ``weight[j]`` (fp32, shared by the heads), or leaves x as it is without a weight.  ``gate`` and
-    ``out`` may be wider buffers; ``act`` is silu or sigmoid."""
+    ``weight[j]`` (fp32 ``[vdim]``, shared by the heads) or ``weight[h vdim + j]`` (fp32 ``[heads * vdim]``),
+    or leaves x as it is without a weight.  ``gate`` and ``out`` may be wider buffers; ``act`` is silu or
+    sigmoid; without a ``gate`` the rows are only normed and multiplied."""
     rows = x.shape[0]
-    if x.shape != (rows, heads * vdim) or gate.dim() != 2 or gate.shape[0] != rows or out.dim() != 2 \
-            or out.shape[0] != rows or not 0 <= gate_off <= gate.shape[1] - heads * vdim \
-            or not 0 <= out_off <= out.shape[1] - heads * vdim:
-        raise KernelError(f"head_norm_gate: x {tuple(x.shape)}, gate {tuple(gate.shape)}, out {tuple(out.shape)} do not fit")
-    if weight is not None and (weight.shape != (vdim,) or weight.dtype != torch.float32):
-        raise KernelError("head_norm_gate: the weight is fp32, one value per element of a head")
-    if activation not in HEAD_GATES:
+    if x.shape != (rows, heads * vdim) or out.dim() != 2 \
+            or out.shape[0] != rows or not 0 <= out_off <= out.shape[1] - heads * vdim:
+        raise KernelError(f"head_norm_gate: x {tuple(x.shape)} and out {tuple(out.shape)} do not fit")
+    if gate is not None and (gate.dim() != 2 or gate.shape[0] != rows or not 0 <= gate_off <= gate.shape[1] - heads * vdim):
+        raise KernelError(f"head_norm_gate: x {tuple(x.shape)} and gate {tuple(gate.shape)} do not fit")
+    if weight is not None and (weight.shape not in ((vdim,), (heads * vdim,)) or weight.dtype != torch.float32):
+        raise KernelError("head_norm_gate: the weight is fp32, one value per element of a head (shared or not)")
+    if gate is not None and activation not in HEAD_GATES:
         raise KernelError(f"head_norm_gate: activation {activation!r} is not one of {sorted(HEAD_GATES)}")
+    w_stride = vdim if weight is not None and heads > 1 and weight.shape == (heads * vdim,) else 0
     check(hip_lib().kva_head_norm_gate(
         _dev(out, "out"), dtype_code(out.dtype), out.shape[1], int(out_off), _dev(x, "x"), dtype_code(x.dtype),
-        _opt(weight, "weight"), float(eps), _dev(gate, "gate"), dtype_code(gate.dtype), gate.shape[1], int(gate_off),
-        rows, heads, vdim, HEAD_GATES[activation], float(mul), _stream()), "head_norm_gate")
+        _opt(weight, "weight"), float(eps), _opt(gate, "gate"), dtype_code(gate.dtype) if gate is not None else 0,
+        gate.shape[1] if gate is not None else 0, int(gate_off),
+        rows, heads, vdim, HEAD_GATES.get(activation, 0), float(mul), w_stride, _stream()), "head_norm_gate")
     return out
 
 
 # --------------------------------------------------------------------------------------
 # Routed experts.
 MOE_TILE = 16
-EXPERT_ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2, "gelu": 3}
+EXPERT_ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2, "gelu": 3, "swish_clamped": 4}     # the last one gated only, with a limit
 
 
 def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, idx: torch.Tensor,
-              wgt: torch.Tensor, renormalise: bool = False, over_chosen: bool = False) -> None:
+              wgt: torch.Tensor, renormalise: bool = False, over_chosen: bool = False, *, scores: str = "softmax",
+              groups: int = 1, keep_groups: int = 1, group_top: int = 2, weight_scale: float = 1.0,
+              sum_eps: float = 0.0) -> None:
     """``scores = softmax(logits)`` over all router outputs; the ``top`` largest of ``scores +
     correction`` are chosen (of equal ones the lowest index) into ``idx`` ``[T, top]``; ``wgt`` gets their
     plain scores, divided by their sum with ``renormalise``.  ``over_chosen``: the ``top`` largest
-    logits (plus correction) are chosen and the weights are the softmax over the chosen logits alone."""
+    logits (plus correction) are chosen and the weights are the softmax over the chosen logits alone.
+    ``scores="sigmoid"``: every output's score is its own ``sigmoid(logit)``.  ``groups`` > 1: the outputs form
+    that many equal runs of neighbours; a run's score is the sum of its ``group_top`` largest ``scores +
+    correction``, and only outputs of the ``keep_groups`` best runs can be chosen.  With ``renormalise`` the
+    weights are ``score / (sum + sum_eps) * weight_scale``, without it ``score * weight_scale``."""
     tokens, outputs = logits.shape
+    if scores not in ("softmax", "sigmoid"):
+        raise KernelError(f"moe_route: scores {scores!r} is neither 'softmax' nor 'sigmoid'")
     if logits.dtype != torch.float32 or idx.shape != (tokens, top) or wgt.shape != (tokens, top) \
             or (correction is not None and correction.shape != (outputs,)):
         raise KernelError(f"moe_route: logits {tuple(logits.shape)}, idx {tuple(idx.shape)}, wgt {tuple(wgt.shape)} do not fit")
     check(hip_lib().kva_moe_route(_dev(idx, "idx", torch.int32), _dev(wgt, "wgt", torch.float32), _dev(logits, "logits"),
                                   _opt(correction, "correction", torch.float32), tokens, outputs, int(top),
-                                  1 if renormalise else 0, 1 if over_chosen else 0, _stream()), "moe_route")
+                                  1 if renormalise else 0, 1 if over_chosen else 0, 1 if scores == "sigmoid" else 0,
+                                  int(groups), int(keep_groups), int(group_top), float(weight_scale), float(sum_eps),
+                                  _stream()), "moe_route")
 
 
 def moe_tiles(slots: int, experts: int) -> int:
@@ -1581,7 +1740,7 @@ def moe_align(idx: torch.Tensor, experts: int, sorted_slot: torch.Tensor, tile_e
 
 def moe_expert_rows(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, sorted_slot: torch.Tensor,
                     tile_expert: torch.Tensor, top: int, *, activation: Optional[str] = None,
-                    slot_weight: Optional[torch.Tensor] = None, gated: bool = False) -> torch.Tensor:
+                    slot_weight: Optional[torch.Tensor] = None, gated: bool = False, limit: float = 0.0) -> torch.Tensor:
     """One product per tile against its expert's matrix ``w[e]`` ``[N, K]``.  With an ``activation``
     (the first product): row ``slot // top`` of ``x`` ``[T, K]``, activated, goes to the slot's sorted
     place of ``out`` ``[places, N]`` (x's type).  With ``slot_weight`` (the second): the row at the
@@ -1610,7 +1769,7 @@ def moe_expert_rows(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, sorted_
         _dev(out, "out"), dtype_code(out.dtype), _dev(x, "x"), _dev(w, "w"), dtype_code(x.dtype),
         _dev(sorted_slot, "sorted_slot", torch.int32), _dev(tile_expert, "tile_expert", torch.int32),
         _opt(slot_weight, "slot_weight"), tiles, int(top), w.shape[1], w.shape[2], 0 if activation is not None else 1,
-        EXPERT_ACTIVATIONS.get(activation, 0), 1 if gated else 0, _stream()), "moe_expert_rows")
+        EXPERT_ACTIVATIONS.get(activation, 0), 1 if gated else 0, float(limit), _stream()), "moe_expert_rows")
     return out
 
 
@@ -1643,10 +1802,14 @@ def small_product_f32(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias:
 
 
 def moe_combine(x: torch.Tensor, rows: torch.Tensor, idx: torch.Tensor, wgt: torch.Tensor, experts: int,
-                out: torch.Tensor, extra: Optional[torch.Tensor] = None) -> torch.Tensor:
+                out: torch.Tensor, extra: Optional[torch.Tensor] = None,
+                extra_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``out[t] = sum over the token's choices`` of the slot's row of ``rows`` (fp32 ``[T * top, width]``,
     already weighted) or, for a choice past the real ``experts`` (an identity expert), ``wgt * x[t]``;
-    ``extra`` (x's shape and type: what an expert that every token uses returned) is added last."""
+    ``extra`` (x's shape and type: what an expert that every token uses returned) is added last - times
+    ``sigmoid(extra_gate[t])`` with ``extra_gate`` (fp32, one number a token)."""
+    if extra_gate is not None and (extra is None or extra_gate.numel() != x.shape[0] or extra_gate.dtype != torch.float32):
+        raise KernelError("moe_combine: the addend's gate is fp32, one number a token")
     tokens, width = x.shape
     top = idx.shape[1]
     if out.shape != x.shape or out.dtype != x.dtype or rows.shape != (tokens * top, width) or rows.dtype != torch.float32 \
@@ -1655,7 +1818,7 @@ def moe_combine(x: torch.Tensor, rows: torch.Tensor, idx: torch.Tensor, wgt: tor
         raise KernelError(f"moe_combine: x {tuple(x.shape)}, rows {tuple(rows.shape)}, idx {tuple(idx.shape)} do not fit")
     check(hip_lib().kva_moe_combine(_dev(out, "out"), _dev(x, "x"), dtype_code(x.dtype), _dev(rows, "rows"),
                                     _dev(idx, "idx", torch.int32), _dev(wgt, "wgt", torch.float32), _opt(extra, "extra"),
-                                    tokens, width, top, int(experts), _stream()), "moe_combine")
+                                    _opt(extra_gate, "extra_gate"), tokens, width, top, int(experts), _stream()), "moe_combine")
     return out
 
 

@@ -47,9 +47,9 @@ _HIP_SIGNATURES = {
     "kva_latent_attention_rowwise": [P, P, P, P, I, P, P, I, I, I, I, I, F, I, I, P, I, P],
     "kva_layernorm": [P, P, I, P, I, P, I, P, I, P, P, I, P, I, I, F, I, F, P],
     "kva_stream_join": [P, I, P, I, P, I, P, I, P, I, I, I, I, P],
-    "kva_act_mul": [P, P, I, I, I, I, P],
+    "kva_act_mul": [P, P, I, I, I, F, I, P],
     "kva_head_gate": [P, P, I, I, I, I, I, P],
-    "kva_qk_encode_cache": [P, I, I, I, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, P, P, P],
+    "kva_qk_encode_cache": [P, I, I, I, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, P, P, I, P],
     "kva_latent_encode_cache": [P, I, I, P, P, P, I, P, I, F, P, P, P, P, I, I, I, I, I, I, I, P],
     "kva_latent_attention_mfma_supported": [I, I, I],
     "kva_attention_rows_mfma_supported": [I, I, I],
@@ -91,17 +91,24 @@ _HIP_SIGNATURES = {
     "kva_host_memory_is_mapped": [P],
     "kva_sample": [P, P, I, I, I, P, P, F, P, U, P, P, I, P, P, P, P, P],
     "kva_mark_tokens": [P, P, P, I, I, P],
-    "kva_causal_conv_act": [P, I, P, I, I, I, P, I, P, LL, I, P, P, I, I, I, I, P],
+    "kva_causal_conv_act": [P, I, P, I, I, I, P, I, P, LL, I, P, P, I, I, I, I, P, P, I, P],
     "kva_gated_delta_rule": [P, P, LL, I, P, I, P, I, I, I, I, P, P, F, P, I, P, P, I, I, I, I, I, P],
     "kva_gated_linear_attention": [P, P, LL, I, P, I, I, I, I, I, P, I, F, P, I, P, P, I, I, I, I, P],
-    "kva_head_norm_gate": [P, I, I, I, P, I, P, F, P, I, I, I, I, I, I, I, F, P],
-    "kva_moe_route": [P, P, P, P, I, I, I, I, I, P],
+    "kva_head_norm_gate": [P, I, I, I, P, I, P, F, P, I, I, I, I, I, I, I, F, I, P],
+    "kva_moe_route": [P, P, P, P, I, I, I, I, I, I, I, I, I, F, F, P],
     "kva_moe_align": [P, P, P, I, I, I, I, P],
-    "kva_moe_expert_rows": [P, I, P, P, I, P, P, P, I, I, I, I, I, I, I, P],
-    "kva_moe_combine": [P, P, I, P, P, P, P, I, I, I, I, P],
+    "kva_moe_expert_rows": [P, I, P, P, I, P, P, P, I, I, I, I, I, I, I, F, P],
+    "kva_moe_combine": [P, P, I, P, P, P, P, P, I, I, I, I, P],
     "kva_small_product_f32": [P, P, I, I, P, I, I, I, I, P, F, P, I, P],
     "kva_norm_into_stream": [P, I, P, I, P, I, P, I, I, I, F, P],
     "kva_table_gate": [P, P, I, P, I, I, I, I, P, P, I, I, I, P],
+    "kva_bias_act": [P, P, I, P, I, I, I, P],
+    "kva_hyper_step": [P, I, P, I, P, P, F, P, P, P, I, F, P, I, P, I, I, P],
+    "kva_hyper_fill": [P, P, I, I, I, I, P],
+    "kva_block_gates": [P, P, P, I, I, I, P, P, I, P, P, P, P],
+    "kva_linear_scan_gate": [P, I, I, I, P, P, I, P, I, I, I, P, P, LL, I, P, P, I, F, P],
+    "kva_matrix_memory_state": [I, I, I],
+    "kva_matrix_memory": [P, P, LL, I, P, I, I, I, I, I, P, F, F, P, P, I, I, I, I, P],
 }
 
 

@@ -194,10 +194,16 @@ class GatedGQAAttention(ProjectedMixer):
     def __init__(self, prefix: str, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  scale: float, position: PartSpec, value_dim: Optional[int] = None, window: int = 0,
                  keep_first: int = 0, bias: bool = False, gate: Optional[str] = "sigmoid",
+                 qk_norm: Optional[str] = None, norm_eps: float = 0.0, sink: bool = False,
                  tensor_names: Optional[Dict[str, str]] = None):
         """``bias``: q, k and v have biases named like their matrices with ``bias_suffix`` added.
-        ``gate``: ``"sigmoid"``, ``"silu"`` or ``None``.  ``tensor_names`` maps ``q k v g o`` and
-        ``bias_suffix`` to names behind ``prefix``."""
+        ``gate``: ``"sigmoid"``, ``"silu"`` or ``None``.  ``qk_norm``: every query and key head passes an
+        RMS norm (``x / sqrt(mean(x^2) + norm_eps) * w`` with a weight of ``head_dim`` elements for the
+        queries and one for the keys, shared by the heads) ``"before_rotation"`` or ``"after_rotation"``;
+        the keys lie in the cache normed and rotated.  ``sink``: a stored number per query head whose
+        exponential is one more term of every softmax denominator (it has no key and no value and is
+        not scaled).  ``tensor_names`` maps ``q k v g o q_norm k_norm sink`` and ``bias_suffix`` to names
+        behind ``prefix``."""
         super().__init__(prefix)
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads is not a multiple of {num_kv_heads} kv heads")
@@ -208,7 +214,11 @@ class GatedGQAAttention(ProjectedMixer):
         self.keep_first = int(keep_first) if self.window > 0 else 0
         self.value_dim = int(head_dim if value_dim is None else value_dim)
         self.bias, self.gate = bool(bias), gate
-        names = dict(q="q", k="k", v="v", g="g", o="o", bias_suffix=".b")
+        if qk_norm not in (None, "before_rotation", "after_rotation"):
+            raise ValueError(f"qk_norm {qk_norm!r} is not one of None, 'before_rotation', 'after_rotation'")
+        self.qk_norm, self.norm_eps, self.sink = qk_norm, float(norm_eps), bool(sink)
+        self.q_weight = self.k_weight = self.sinks = None
+        names = dict(q="q", k="k", v="v", g="g", o="o", bias_suffix=".b", q_norm="q.norm", k_norm="k.norm", sink="sink")
         names.update(tensor_names or {})
         self.bias_suffix = names.pop("bias_suffix")
         self.names = {key: prefix + name for key, name in names.items()}
@@ -225,10 +235,19 @@ class GatedGQAAttention(ProjectedMixer):
         if self.bias:
             for key in "qkv":
                 specs[n[key] + self.bias_suffix] = TensorSpec((specs[n[key]].shape[0],), init="normal", role="vector")
+        if self.qk_norm is not None:
+            specs[n["q_norm"]] = TensorSpec((d,), init="norm", role="vector")
+            specs[n["k_norm"]] = TensorSpec((d,), init="norm", role="vector")
+        if self.sink:
+            specs[n["sink"]] = TensorSpec((self.num_heads,), init="normal", role="vector")
         return specs
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         n = self.names
+        if self.qk_norm is not None:        # norms and the softmax's terms are 32-bit
+            self.q_weight, self.k_weight = tensors[n["q_norm"]].float().contiguous(), tensors[n["k_norm"]].float().contiguous()
+        if self.sink:
+            self.sinks = tensors[n["sink"]].float().contiguous()
         rows = [tensors[n[key]] for key in "qkv"] + ([tensors[n["g"]]] if self.gate is not None else [])
         self._w_in = torch.cat(rows, dim=0).contiguous()
         self._w_out = tensors[n["o"]]
@@ -255,16 +274,18 @@ class GatedGQAAttention(ProjectedMixer):
         cos, sin = self.position.tables(y.device) if hasattr(self.position, "tables") else (None, None)
         K.qk_encode_cache(qkv, batch.positions, self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim,
                           cos, sin, getattr(self.position, "pairing", "half") == "interleaved",
-                          getattr(self.position, "unit_norm_eps", None),
+                          self.norm_eps if self.qk_norm is not None else getattr(self.position, "unit_norm_eps", None),
                           kv.k_cache if write else None, kv.v_cache if write else None,
-                          kv.slot_mapping if write else None, bias=self.qkv_bias)
+                          kv.slot_mapping if write else None, bias=self.qkv_bias, q_weight=self.q_weight,
+                          k_weight=self.k_weight, norm_first=self.qk_norm == "before_rotation")
         direct = self.gate is None and mul == 1.0 and out_col0 == 0 and out.shape[1] == self.inner_width
         heads = out if direct else torch.empty((y.shape[0], self.inner_width), dtype=y.dtype, device=y.device)
         attn_ops.paged_attention(qkv, heads, kv, batch, self.num_heads, self.num_kv_heads, self.head_dim, self.scale,
-                                 self.window, keep_first=self.keep_first, value_dim=self.value_dim)
+                                 self.window, keep_first=self.keep_first, value_dim=self.value_dim, sinks=self.sinks)
         if not direct:
             if self.gate is None:
-                out[:, out_col0:out_col0 + self.inner_width] = heads * mul
+                # the heads times the constant, into their columns of the wider buffer
+                K.head_norm_gate(heads, None, 0.0, None, 0, out, out_col0, self.num_heads, self.value_dim, None, mul)
             else:
                 K.head_norm_gate(heads, None, 0.0, y, col0 + self.qkv_width, out, out_col0, self.num_heads,
                                  self.value_dim, self.gate, mul)

@@ -141,6 +141,9 @@ class MixerContext:
     batch: "object"                       # engine.batch.StepBatch
     kv: Optional[KVView] = None
     state: Optional[torch.Tensor] = None  # [seats, *StateSpec.shape] of this mixer call
+    # the rows a projected mixer's joined input projection read (set by whoever runs that product), for
+    # what a mixer forms from its input in 32-bit beside the projection (the gates of a recurrence)
+    x: Optional[torch.Tensor] = None
 
 
 @dataclass
@@ -188,6 +191,20 @@ class StreamCopy:
     again; whoever wants a pending output treats it as none."""
 
     rows: torch.Tensor
+
+
+@dataclass
+class PendingMix:
+    """A branch output that has not entered a residual stream of several copies yet (hyper-connections:
+    ``x_t <- sum_s mix[s, t] x_s + mult * out_w[t] * y``, all copies at once).  Whoever reads the stream next -
+    the next block, or the model's last norm - does it in the pass that reads (``ops.kernels.hyper_step``).
+    One copy with ``mix = out_w = 1`` is a plain residual stream whose branches enter times ``mult``."""
+
+    y: torch.Tensor
+    mix: torch.Tensor           # fp32 [streams, streams], indexed [from, to]
+    out_w: torch.Tensor         # fp32 [streams]
+    mult: float
+    streams: int
 
 
 @dataclass
@@ -334,6 +351,7 @@ class ProjectedMixer(Mixer):
 
     def forward(self, x: torch.Tensor, ctx: MixerContext) -> torch.Tensor:
         y = self._in(x)
+        ctx.x = x
         inner = torch.empty((x.shape[0], self.inner_width), dtype=x.dtype, device=x.device)
         self.forward_inner(y, 0, ctx, 0, inner, 0, 1.0)
         return self._out(inner)

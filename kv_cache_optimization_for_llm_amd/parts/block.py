@@ -7,14 +7,15 @@ residual kernel would have produced.
 """
 from __future__ import annotations
 
-from typing import Optional
+from typing import Dict, Optional
 
 import torch
 
 from ..config.registry import BLOCKS, LAYER_INPUTS
 from ..models.spec import PartSpec
 from ..ops import kernels as K
-from .base import Block, BranchTail, MixerContext, Norm, NormedRows, PendingSum, StreamCopy
+from ..models.spec import TensorSpec
+from .base import Block, BranchTail, MixerContext, Norm, NormedRows, Part, PendingMix, PendingSum, StreamCopy
 
 
 @BLOCKS.register("pre_norm")
@@ -157,3 +158,93 @@ class PostNormBlock(Block):
         if self.layer_input is not None:
             h = self._into_stream(hidden, self.layer_input.forward(h, ctx), self.layer_input)
         return hidden, (StreamCopy(h) if h is not hidden else None)
+
+
+class HyperConnection(Part):
+    """How one branch reads and re-enters a residual stream of ``streams`` copies: input weights ``in`` [S]
+    (the branch reads ``sum_s in[s] x_s``), a mixing matrix ``mix`` [S, S] indexed [from, to] and output
+    weights ``out`` [S] (``x_t <- sum_s mix[s, t] x_s + mult * out[t] * y``).  ``learned=False``: no tensors,
+    all of them 1 - with one copy that is the plain residual sum."""
+
+    def __init__(self, prefix: str, *, streams: int, learned: bool = True):
+        super().__init__(prefix)
+        self.streams, self.learned = int(streams), bool(learned)
+        if not self.learned and self.streams != 1:
+            raise ValueError(f"{prefix}: several copies of the stream need stored weights")
+        self.in_w = self.out_w = self.mix = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        if not self.learned:
+            return {}
+        S, p = self.streams, self.prefix
+        return {p + "in": TensorSpec((S,), init="norm", role="vector"),
+                p + "out": TensorSpec((S,), init="norm", role="vector"),
+                p + "mix": TensorSpec((S, S), init="eye", role="vector")}
+
+    def load(self, tensors: Dict[str, torch.Tensor], device=None) -> None:
+        if self.learned:
+            p = self.prefix
+            # the stream and every sum into it are 32-bit: so are these
+            self.in_w, self.out_w = tensors[p + "in"].float().contiguous(), tensors[p + "out"].float().contiguous()
+            self.mix = tensors[p + "mix"].float().contiguous()
+        else:
+            self.in_w = self.out_w = torch.ones(1, dtype=torch.float32, device=device)
+            self.mix = torch.ones((1, 1), dtype=torch.float32, device=device)
+
+
+@BLOCKS.register("hyper_connections")
+class HyperConnectionBlock(Block):
+    """Pre-norm branches over a residual stream kept in 32-bit as ``streams`` copies of every row, side by side
+    (``hidden`` is ``[T, streams * width]``): for the mixer and then the feed-forward, ``u = sum_s in[s] x_s``,
+    ``y = branch(norm(u))``, and all copies at once from the old ones ``x_t <- sum_s mix[s, t] x_s + residual_mult
+    * out[t] * y``.  The layer's norms are layer norms (weight and, if they have one, bias) whose arithmetic
+    runs inside the same pass: one launch (``ops.kernels.hyper_step``) lets the previous branch's output into
+    the copies, reads them out and norms - so a layer is two such launches, and the last output travels on as
+    :class:`~.base.PendingMix` to whoever reads the stream next.  ``learned=False`` (one copy, no tensors):
+    ``x <- x + residual_mult * branch(norm(x))``.  A layer without a feed-forward names only the ``"mixer"``
+    norm.  ``connection_names``: the two connections' tensor prefixes behind ``prefix``."""
+
+    graph_safe = True
+    NORM_NAMES = ("mixer", "feed_forward")
+
+    def __init__(self, mixer, feed_forward, norms, *, prefix: str = "", streams: int = 1, learned: bool = True,
+                 residual_mult: float = 1.0, connection_names=("hc1.", "hc2.")):
+        self.has_ffn = not getattr(feed_forward, "absent", False)
+        if not self.has_ffn:
+            self.NORM_NAMES = ("mixer",)
+        super().__init__(mixer, feed_forward, norms)
+        self.streams, self.residual_mult = int(streams), float(residual_mult)
+        self.connections = [HyperConnection(prefix + name, streams=streams, learned=learned)
+                            for name in connection_names[:2 if self.has_ffn else 1]]
+        for norm in self.norms.values():
+            if not getattr(norm, "center", False) or getattr(norm, "weight_offset", 0.0):
+                raise ValueError("this arrangement runs centred layer norms (weight, optional bias) inside its own pass")
+
+    def parts(self):
+        return (*super().parts(), *self.connections)
+
+    def first_norm(self) -> Optional[Norm]:
+        return None
+
+    def _read(self, hidden, pending, connection, norm):
+        """Lets ``pending`` into the copies, then the branch's input: the normed read-out."""
+        if connection.in_w is None or connection.in_w.device != hidden.device:
+            connection.load({}, hidden.device)
+        x = torch.empty((hidden.shape[0], norm.width), dtype=norm.out_dtype or norm.weight.dtype, device=hidden.device)
+        enter = {} if pending is None else dict(y=pending.y, mix=pending.mix, out_w=pending.out_w, mult=pending.mult)
+        return K.hyper_step(hidden, self.streams, in_w=connection.in_w, norm_weight=norm.weight, norm_bias=norm.bias,
+                            eps=norm.eps, out=x, **enter)
+
+    def forward(self, hidden: torch.Tensor, delta, ctx: MixerContext, next_norm: Optional[Norm] = None):
+        if delta is not None and not isinstance(delta, PendingMix):
+            raise TypeError("this arrangement takes the stream's copies and a pending output with its way into them")
+        if hidden.dtype != torch.float32 or hidden.shape[1] != self.streams * self.norms["mixer"].width:
+            raise TypeError(f"the stream must be 32-bit rows of {self.streams} copies")
+        first = self.connections[0]
+        a = self.mixer.forward(self._read(hidden, delta, first, self.norms["mixer"]), ctx)
+        pending = PendingMix(a, first.mix, first.out_w, self.residual_mult, self.streams)
+        if self.has_ffn:
+            second = self.connections[1]
+            f = self.feed_forward.forward(self._read(hidden, pending, second, self.norms["feed_forward"]), ctx)
+            pending = PendingMix(f, second.mix, second.out_w, self.residual_mult, self.streams)
+        return hidden, pending

@@ -92,6 +92,7 @@ class SideBySide(Mixer):
 
     def forward(self, x: torch.Tensor, ctx: MixerContext) -> torch.Tensor:
         y = self.w_in(x)
+        ctx.x = x
         inner = torch.empty((x.shape[0], self.inner_width), dtype=x.dtype, device=x.device)
         for c, col0, out0, soff, scale in zip(self.children, self.col0, self.out_col0, self.state_off, self.scales):
             c.forward_inner(y, col0, ctx, soff, inner, out0, scale)

@@ -39,12 +39,14 @@ class SwiGLU(FeedForward):
     graph_safe = True
 
     def __init__(self, prefix: str, *, hidden_size: int, intermediate_size: int, activation: str = "silu",
-                 tensor_names: Optional[Dict[str, str]] = None):
-        """``tensor_names`` maps ``gate``, ``up``, ``down`` to the matrices' names behind ``prefix``."""
+                 limit: float = 0.0, tensor_names: Optional[Dict[str, str]] = None):
+        """``tensor_names`` maps ``gate``, ``up``, ``down`` to the matrices' names behind ``prefix``.
+        ``activation="swish_clamped"`` with its ``limit``: ``g sigmoid(1.702 g) (u + 1)`` with ``g = min(gate,
+        limit)``, ``u = clamp(up, -limit, limit)``."""
         super().__init__(prefix)
-        if activation not in K.ACTIVATIONS:
-            raise ValueError(f"activation {activation!r} is not one of {sorted(K.ACTIVATIONS)}")
-        self.activation = activation
+        if activation not in K.GATED_ACTIVATIONS:
+            raise ValueError(f"activation {activation!r} is not one of {sorted(K.GATED_ACTIVATIONS)}")
+        self.activation, self.limit = activation, float(limit)
         names = dict(gate="gate_proj.weight", up="up_proj.weight", down="down_proj.weight")
         names.update(tensor_names or {})
         self.names = {key: prefix + name for key, name in names.items()}
@@ -61,7 +63,9 @@ class SwiGLU(FeedForward):
         g, u = tensors[self.names["gate"]], tensors[self.names["up"]]
         if g.dtype != u.dtype:
             raise ValueError(f"{p}: gate and up projection weights are stored in different dtypes")
-        self.gate_up = Linear(torch.cat([g, u], dim=0), halves=2)
+        # (the tiled copy of a joined matrix pairs gate and up rows for the products that activate in their
+        # epilogue; an activation that runs as its own kernel reads the plain product's two halves)
+        self.gate_up = Linear(torch.cat([g, u], dim=0), halves=2 if self.activation in K.ACTIVATIONS else 1)
         self.down = Linear(tensors[self.names["down"]])
 
     fuses_tail = True
@@ -74,7 +78,8 @@ class SwiGLU(FeedForward):
         """``x`` may be NormedRows; with a ``tail`` the down projection adds into the residual
         stream and prepares the next norm when the shapes allow (NormedRows are returned)."""
         rows = x.shape[0]
-        up_kernel = self.gate_up.fused_kernel(rows, x.dtype)
+        # (the products' epilogues know the plain activations; a clamped one runs as its own kernel)
+        up_kernel = self.gate_up.fused_kernel(rows, x.dtype) if self.activation in K.ACTIVATIONS else None
         # Both products in their few-rows form and at most 16 rows: the activations go from one to
         # the other in the order the second one's lanes read them (ops.kernels.TiledRows).
         tiled = (up_kernel == Linear.FEW_ROWS and rows <= K.TiledRows.MAX_ROWS and self.intermediate_size % 8 == 0
@@ -89,7 +94,7 @@ class SwiGLU(FeedForward):
         elif self.activation == "silu":
             K.silu_mul(self.gate_up(x), act)
         else:
-            K.act_mul(self.gate_up(x), act, self.activation)
+            K.act_mul(self.gate_up(x), act, self.activation, self.limit)
         if tail is not None:
             fused = self.down.into_residual(act, tail)
             if fused is not None:
@@ -97,3 +102,39 @@ class SwiGLU(FeedForward):
         if tiled:
             act = act.to_rows()
         return self.down(act)
+
+
+@FEED_FORWARDS.register("mlp")
+class PlainMLP(FeedForward):
+    """A feed-forward that is not gated: ``down(act(up(x)))`` without biases; ``act`` one of silu, relu,
+    gelu_tanh, applied by its own kernel between the two products."""
+
+    graph_safe = True
+
+    def __init__(self, prefix: str, *, hidden_size: int, intermediate_size: int, activation: str = "gelu_tanh",
+                 tensor_names: Optional[Dict[str, str]] = None):
+        """``tensor_names`` maps ``up``, ``down`` to the matrices' names behind ``prefix``."""
+        super().__init__(prefix)
+        if activation not in K.ACTIVATIONS:
+            raise ValueError(f"activation {activation!r} is not one of {sorted(K.ACTIVATIONS)}")
+        self.activation = activation
+        names = dict(up="up", down="down")
+        names.update(tensor_names or {})
+        self.names = {key: prefix + name for key, name in names.items()}
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.up: Optional[Linear] = None
+        self.down: Optional[Linear] = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        n, h, i = self.names, self.hidden_size, self.intermediate_size
+        return {n["up"]: TensorSpec((i, h)), n["down"]: TensorSpec((h, i))}
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.up, self.down = Linear(tensors[self.names["up"]]), Linear(tensors[self.names["down"]])
+
+    def activation_elements(self) -> int:
+        return 2 * self.intermediate_size + self.hidden_size
+
+    def forward(self, x, ctx: MixerContext, tail: Optional[BranchTail] = None):
+        z = self.up(x)
+        return self.down(K.bias_act(z, z, self.activation))

@@ -41,11 +41,32 @@ class RoutedExperts(FeedForward):
     def __init__(self, prefix: str, *, hidden_size: int, intermediate_size: int, experts: int, top: int,
                  identity: int = 0, activation: str = "gelu", correction: bool = True, renormalise: bool = False,
                  gated: bool = False, router_bias: bool = False, softmax_over: str = "all",
-                 shared_intermediate: int = 0, tensor_names: Optional[Dict[str, str]] = None):
-        """``tensor_names`` maps ``router``, ``router_bias``, ``correction``, ``gate``, ``up``, ``down`` and
-        ``shared`` (a prefix) to names behind ``prefix``; the experts' names hold ``{e}`` for the expert's
-        number."""
+                 shared_intermediate: int = 0, scores: str = "softmax", groups: int = 1, keep_groups: int = 1,
+                 group_top: int = 2, weight_scale: float = 1.0, sum_eps: float = 0.0, limit: float = 0.0,
+                 shared_limit: Optional[float] = None, shared_gate: bool = False,
+                 tensor_names: Optional[Dict[str, str]] = None):
+        """``scores="sigmoid"``: every router output's score is its own sigmoid.  ``groups`` > 1: the outputs
+        form so many equal runs of neighbours, a run's score is the sum of its ``group_top`` largest choice
+        scores (score + correction), and only outputs of the ``keep_groups`` best runs can be chosen.
+        ``weight_scale`` multiplies the weights; ``sum_eps`` is added to the sum they are divided by
+        (``renormalise``).  ``activation="swish_clamped"`` (gated experts) with ``limit``: ``g sigmoid(1.702 g)
+        (u + 1)``, ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``; ``shared_limit``: the limit of the
+        expert every token uses (default: ``limit``).  ``shared_gate``: that expert's result enters times
+        ``sigmoid(w . x)``, one number a token, ``w`` stored as ``[1, hidden]``.
+        ``tensor_names`` maps ``router``, ``router_bias``, ``correction``, ``gate``, ``up``, ``down``,
+        ``shared`` (a prefix) and ``shared_gate`` to names behind ``prefix``; the experts' names hold ``{e}`` for
+        the expert's number."""
         super().__init__(prefix)
+        if scores not in ("softmax", "sigmoid"):
+            raise ValueError(f"{prefix}: scores {scores!r} is neither 'softmax' nor 'sigmoid'")
+        self.scores, self.groups, self.keep_groups, self.group_top = scores, int(groups), int(keep_groups), int(group_top)
+        self.weight_scale, self.sum_eps, self.limit = float(weight_scale), float(sum_eps), float(limit)
+        self.shared_limit = self.limit if shared_limit is None else float(shared_limit)
+        self.has_shared_gate = bool(shared_gate)
+        if self.groups < 1 or not 1 <= self.keep_groups <= self.groups or (int(experts) + int(identity)) % self.groups:
+            raise ValueError(f"{prefix}: {groups} groups (of which {keep_groups} are kept) do not divide the router's outputs")
+        if activation == "swish_clamped" and not gated:
+            raise ValueError(f"{prefix}: the clamped activation is a gated one")
         if softmax_over not in ("all", "chosen"):
             raise ValueError(f"{prefix}: softmax_over {softmax_over!r} is neither 'all' nor 'chosen'")
         self.gated, self.has_router_bias, self.over_chosen = bool(gated), bool(router_bias), softmax_over == "chosen"
@@ -58,18 +79,20 @@ class RoutedExperts(FeedForward):
             raise ValueError(f"activation {activation!r} is not one of {sorted(K.EXPERT_ACTIVATIONS)}")
         self.activation, self.has_correction, self.renormalise = activation, bool(correction), bool(renormalise)
         names = dict(router="router", router_bias="router.b", correction="correction", gate="e{e}.gate", up="e{e}.up",
-                     down="e{e}.down", shared="shared.")
+                     down="e{e}.down", shared="shared.", shared_gate="shared.sg")
         names.update(tensor_names or {})
         self.names = {key: prefix + name for key, name in names.items()}
         self.outputs = self.experts + self.identity
         self.shared = None
         if self.shared_intermediate > 0:
-            if activation not in K.ACTIVATIONS:
-                raise ValueError(f"{prefix}: the expert every token uses runs with one of {sorted(K.ACTIVATIONS)}")
+            if activation not in K.GATED_ACTIVATIONS:
+                raise ValueError(f"{prefix}: the expert every token uses runs with one of {sorted(K.GATED_ACTIVATIONS)}")
             from .mlp import SwiGLU
             self.shared = SwiGLU(self.names["shared"], hidden_size=self.hidden_size,
                                  intermediate_size=self.shared_intermediate, activation=activation,
-                                 tensor_names=dict(gate="gate", up="up", down="down"))
+                                 limit=self.shared_limit, tensor_names=dict(gate="gate", up="up", down="down"))
+        if self.has_shared_gate and self.shared is None:
+            raise ValueError(f"{prefix}: a gate without the expert every token uses")
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         n, W, I = self.names, self.hidden_size, self.intermediate_size
@@ -85,6 +108,8 @@ class RoutedExperts(FeedForward):
             specs[n["down"].format(e=e)] = TensorSpec((W, I))
         if self.shared is not None:
             specs.update(self.shared.tensor_specs())
+        if self.has_shared_gate:
+            specs[n["shared_gate"]] = TensorSpec((1, W))
         return specs
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
@@ -94,6 +119,7 @@ class RoutedExperts(FeedForward):
         self.router_bias = tensors[n["router_bias"]].float().contiguous() if self.has_router_bias else None
         if self.shared is not None:
             self.shared.load(tensors)
+        self.shared_gate = tensors[n["shared_gate"]].contiguous() if self.has_shared_gate else None
         if self.experts and self.gated:
             # rows 2 j and 2 j + 1 of an expert's first matrix: output j's gate row and its up row
             ups = []
@@ -118,7 +144,9 @@ class RoutedExperts(FeedForward):
                                      bias=self.router_bias)
         idx = torch.empty((T, self.top), dtype=torch.int32, device=dev)
         wgt = torch.empty((T, self.top), dtype=torch.float32, device=dev)
-        K.moe_route(logits, self.correction, self.top, idx, wgt, self.renormalise, over_chosen=self.over_chosen)
+        K.moe_route(logits, self.correction, self.top, idx, wgt, self.renormalise, over_chosen=self.over_chosen,
+                    scores=self.scores, groups=self.groups, keep_groups=self.keep_groups, group_top=self.group_top,
+                    weight_scale=self.weight_scale, sum_eps=self.sum_eps)
         if RoutedExperts.on_route is not None and not torch.cuda.is_current_stream_capturing():
             RoutedExperts.on_route(self, idx)
         slots = T * self.top
@@ -130,8 +158,11 @@ class RoutedExperts(FeedForward):
             K.moe_align(idx, self.experts, sorted_slot, tile_expert)
             act = torch.empty((tiles * K.MOE_TILE, self.intermediate_size), dtype=x.dtype, device=dev)
             K.moe_expert_rows(x, self.w_up, act, sorted_slot, tile_expert, self.top, activation=self.activation,
-                              gated=self.gated)
+                              gated=self.gated, limit=self.limit)
             K.moe_expert_rows(act, self.w_down, rows, sorted_slot, tile_expert, self.top, slot_weight=wgt)
         out = torch.empty_like(x)
         extra = self.shared.forward(x, ctx) if self.shared is not None else None
-        return K.moe_combine(x, rows, idx, wgt, self.experts, out, extra=extra)
+        gate = None
+        if self.shared_gate is not None:        # one number a token, in 32-bit; its sigmoid is taken where the rows are added
+            gate = K.small_product_f32(x, self.shared_gate, torch.empty((T, 1), dtype=torch.float32, device=dev))
+        return K.moe_combine(x, rows, idx, wgt, self.experts, out, extra=extra, extra_gate=gate)

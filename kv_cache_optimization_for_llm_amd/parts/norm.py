@@ -12,7 +12,7 @@ import torch
 from ..config.registry import NORMS
 from ..models.spec import TensorSpec
 from ..ops import kernels as K
-from .base import Norm
+from .base import Norm, PendingMix
 
 
 @NORMS.register("rmsnorm")
@@ -53,7 +53,7 @@ class RMSNorm(Norm):
 @NORMS.register("layernorm")
 class LayerNorm(Norm):
     """``y = (x - mean) / sqrt(var + eps) * w`` with the variance as the mean of the squared
-    deviations; a weight, no bias.  Statistics are fp32.  The rows it reads may be an fp32 stream
+    deviations; a weight and, optionally, a bias.  Statistics are fp32.  The rows it reads may be an fp32 stream
     while it writes ``out_dtype`` rows (the type the products behind it take).  ``delta`` may be one
     branch output or a tuple of two: they are added to ``x`` in place first.  ``forward_pair``
     writes two normalised copies, this norm's and a ``twin``'s (same width and eps, another
@@ -62,22 +62,39 @@ class LayerNorm(Norm):
     graph_safe = True
 
     def __init__(self, prefix: str, *, width: int, eps: float, weight_name: str = "weight",
-                 out_dtype: Optional[str] = None, center: bool = True, weight_offset: float = 0.0):
+                 out_dtype: Optional[str] = None, center: bool = True, weight_offset: float = 0.0,
+                 bias_name: Optional[str] = None, streams: int = 1):
         """``center=False``: the mean is not taken off (``x / sqrt(mean(x^2) + eps) * w``, an RMS norm
         over a stream of another type than the products').  ``weight_offset``: the weight is stored
-        around zero and multiplies as ``weight_offset + w`` (the sum is formed once, in 32-bit)."""
+        around zero and multiplies as ``weight_offset + w`` (the sum is formed once, in 32-bit).
+        ``bias_name``: the norm has a bias, ``... * w + b``.  ``streams``: the rows it reads hold so
+        many copies of the stream side by side (32-bit), and what is normed is their sum; a pending
+        :class:`~.base.PendingMix` enters the copies first.  A norm with a bias or over several copies
+        reads a 32-bit stream (``ops.kernels.hyper_step``)."""
         super().__init__(prefix)
         self.width, self.eps = int(width), float(eps)
         self.weight_name = prefix + weight_name
+        self.bias_name = None if bias_name is None else prefix + bias_name
+        self.streams = int(streams)
+        if (self.bias_name is not None or self.streams > 1) and (not center or weight_offset):
+            raise ValueError(f"{prefix}: a bias or several copies of the stream go with the plain centred form")
+        self.bias: Optional[torch.Tensor] = None
+        self._ones: Optional[torch.Tensor] = None
         self.out_dtype = {None: None, "bfloat16": torch.bfloat16, "float32": torch.float32}[out_dtype]
         self.center, self.weight_offset = bool(center), float(weight_offset)
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        return {self.weight_name: TensorSpec((self.width,), init="zeros" if self.weight_offset else "norm", role="vector")}
+        specs = {self.weight_name: TensorSpec((self.width,), init="zeros" if self.weight_offset else "norm", role="vector")}
+        if self.bias_name is not None:
+            specs[self.bias_name] = TensorSpec((self.width,), init="normal", role="vector")
+        return specs
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.weight = tensors[self.weight_name].contiguous()
+        if self.bias_name is not None:
+            self.bias = tensors[self.bias_name].contiguous()
+        self._ones = torch.ones(self.streams, dtype=torch.float32, device=self.weight.device)
         if self.weight_offset:
             if self.out_dtype is None:
                 self.out_dtype = self.weight.dtype          # the products behind the norm take the stored type
@@ -103,6 +120,14 @@ class LayerNorm(Norm):
 
     def forward(self, x, out=None, delta=None, row_idx=None):
         out = self._out(x, row_idx) if out is None else out
+        if self.bias is not None or self.streams > 1 or isinstance(delta, PendingMix):
+            if delta is not None and not isinstance(delta, PendingMix):
+                raise TypeError(f"{self.prefix}: this norm takes a pending output with its way into the stream's copies")
+            if delta is not None and delta.streams != self.streams:
+                raise ValueError(f"{self.prefix}: the pending output belongs to a stream of {delta.streams} copies")
+            enter = {} if delta is None else dict(y=delta.y, mix=delta.mix, out_w=delta.out_w, mult=delta.mult)
+            return K.hyper_step(x, self.streams, in_w=self._ones, norm_weight=self.weight, norm_bias=self.bias,
+                                eps=self.eps, out=out, row_idx=row_idx, **enter)
         return K.layernorm(x, self.weight, self.eps, out, deltas=self._deltas(delta), row_idx=row_idx,
                            rms=not self.center, delta_scale=self._scale(delta))
 

@@ -19,6 +19,11 @@ order of every sum depends on the sizes alone.
 * :class:`LightningAttention` (``"lightning_attention"``): ``S_t = decay_h S_(t-1) + k_t v_t^T``,
   ``o_t = S_t^T q_t`` with one fixed decay a head, silu on q, k and v, and ONE norm over all heads'
   read-outs together.
+* :class:`MatrixMemory` (``"matrix_memory"``): a matrix ``S``, a vector ``n`` and a running maximum ``m``
+  per head under exponential input and forget gates: ``m' = max(f + m, i)``, ``S <- e^(f + m - m') S +
+  e^(i - m') k v^T``, ``n`` likewise with ``k`` alone, ``o = S^T q / (max(|n . q|, e^(-m')) + 1e-6)``.
+* :class:`RealGatedLRU` (``"real_gated_lru"``): per channel ``S_t = a_t S_(t-1) + sqrt(1 - a_t^2) i_t u_t``
+  behind a short causal convolution, with gates made by block-diagonal matrices, times a gelu branch.
 """
 from __future__ import annotations
 
@@ -311,3 +316,157 @@ class LightningAttention(ProjectedMixer):
         # one norm over all the heads' read-outs: a single "head" as wide as the row
         K.head_norm_gate(o, self.norm_weight, self.norm_eps, y, col0 + self.g_off, out, out_col0, 1, self.inner_width,
                          self.gate, mul)
+
+
+@MIXERS.register("matrix_memory")
+class MatrixMemory(ProjectedMixer):
+    """A matrix memory with exponential gates.  Per head: ``q = W_q x * query_scale`` (default ``head_dim^-1/2``),
+    ``k = W_k x`` (``head_dim``), ``v = W_v x`` (``value_dim``); a log input gate ``i = cap tanh((W_i x + b_i) /
+    cap)`` and a log forget gate ``f = logsigmoid(cap tanh((W_f x + b_f) / cap))``; with a running maximum m
+    (0 at a request's start, like S and n): ``m' = max(f + m, i)``, ``S <- e^(f + m - m') S + e^(i - m') k v^T``,
+    ``n <- e^(f + m - m') n + e^(i - m') k``, ``o = S^T q / (max(|n . q|, e^(-m')) + 1e-6)``.  Every head's
+    read-out is divided by its root mean square, the heads are joined and multiplied by a weight of all
+    heads' size and by ``gate(W_g x)``, then projected.  The gates' inputs are formed in 32-bit from the
+    mixer's input rows (a product of their own, not columns of the joined projection); S, n and m are fp32
+    in the seat's state row."""
+
+    graph_safe = True
+
+    def __init__(self, prefix: str, *, hidden_size: int, num_heads: int, head_dim: int, value_dim: int, gate_cap: float,
+                 norm_eps: float, query_scale: Optional[float] = None, gate: str = "sigmoid",
+                 tensor_names: Optional[Dict[str, str]] = None):
+        """``tensor_names`` maps ``q k v g o norm i f i_bias f_bias`` to names behind ``prefix``."""
+        super().__init__(prefix)
+        if gate not in K.HEAD_GATES:
+            raise ValueError(f"{prefix}: gate {gate!r} is not one of {sorted(K.HEAD_GATES)}")
+        if not gate_cap > 0:
+            raise ValueError(f"{prefix}: gate_cap {gate_cap} must be positive")
+        self.hidden_size, self.num_heads, self.head_dim, self.value_dim = int(hidden_size), int(num_heads), int(head_dim), int(value_dim)
+        self.gate_cap, self.norm_eps, self.gate = float(gate_cap), float(norm_eps), gate
+        self.query_scale = float(head_dim) ** -0.5 if query_scale is None else float(query_scale)
+        self.inner_width = self.num_heads * self.value_dim
+        self.names = _names(dict(q="q", k="k", v="v", g="g", o="o", norm="norm", i="i", f="f", i_bias="i.b", f_bias="f.b"),
+                            tensor_names, prefix)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        n, W, H, hd, hv = self.names, self.hidden_size, self.num_heads, self.num_heads * self.head_dim, self.inner_width
+        return {n["q"]: TensorSpec((hd, W)), n["k"]: TensorSpec((hd, W)), n["v"]: TensorSpec((hv, W)),
+                n["g"]: TensorSpec((hv, W)), n["o"]: TensorSpec((W, hv)),
+                n["norm"]: TensorSpec((hv,), init="norm", role="vector"),
+                n["i"]: TensorSpec((H, W)), n["f"]: TensorSpec((H, W)),
+                n["i_bias"]: TensorSpec((H,), init="normal", role="vector"),
+                n["f_bias"]: TensorSpec((H,), init="normal", role="vector")}
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        t = {key: tensors[name] for key, name in self.names.items()}
+        self._w_in = torch.cat([t["q"], t["k"], t["v"], t["g"]], dim=0).contiguous()
+        self._w_out = t["o"]
+        hd, hv = self.num_heads * self.head_dim, self.inner_width
+        self.q_off, self.k_off, self.v_off, self.g_off = 0, hd, 2 * hd, 2 * hd + hv
+        self.gate_weight = torch.cat([t["i"], t["f"]], dim=0).contiguous()                     # [2 heads, hidden]: zi, then zf
+        self.gate_bias = torch.cat([t["i_bias"], t["f_bias"]]).float().contiguous()
+        self.norm_weight = t["norm"].float().contiguous()
+        self.load_projections()
+
+    def input_weight(self) -> torch.Tensor:
+        return self._w_in
+
+    def output_weight(self) -> torch.Tensor:
+        return self._w_out
+
+    def state_elements(self) -> int:
+        # S of every head, then n and m as the kernel lays them out (a copy per run of 16 value columns)
+        tiles = -(-self.value_dim // 16)
+        return self.num_heads * self.head_dim * self.value_dim + self.num_heads * tiles * (self.head_dim + 1)
+
+    def activation_elements(self) -> int:
+        return 2 * self.num_heads * self.head_dim + 5 * self.inner_width + self.hidden_size
+
+    def forward_inner(self, y, col0, ctx: MixerContext, state_off, out, out_col0, mul) -> None:
+        batch, T = ctx.batch, y.shape[0]
+        if ctx.x is None:
+            raise K.KernelError(f"{self.prefix}: the gates are formed from the mixer's input rows, which were not handed on")
+        if self.state_elements() != K.matrix_memory_state(self.num_heads, self.head_dim, self.value_dim):
+            raise K.KernelError(f"{self.prefix}: the kernel lays the state out differently")
+        gates = K.small_product_f32(ctx.x, self.gate_weight,
+                                    torch.empty((T, 2 * self.num_heads), dtype=torch.float32, device=y.device),
+                                    bias=self.gate_bias)
+        o = torch.empty((T, self.inner_width), dtype=torch.float32, device=y.device)
+        K.matrix_memory(y, col0 + self.q_off, col0 + self.k_off, col0 + self.v_off, gates, self.gate_cap, self.query_scale,
+                        o, ctx.state, state_off, batch.entry_q_start, batch.entry_seat, self.num_heads, self.head_dim,
+                        self.value_dim)
+        K.head_norm_gate(o, self.norm_weight, self.norm_eps, y, col0 + self.g_off, out, out_col0, self.num_heads,
+                         self.value_dim, self.gate, mul)
+
+
+@MIXERS.register("real_gated_lru")
+class RealGatedLRU(ProjectedMixer):
+    """A recurrent block around a real-gated linear recurrent unit.  Two branches of ``width`` channels read
+    the input: ``y = gelu_tanh(W_y x + b_y)`` and ``u = conv(W_x x + b_x)``, a causal convolution per channel
+    over ``conv_taps`` tokens (weight ``[channels, taps]``, the last column the current token's; a bias; no
+    activation; zeros before a request's start).  The channels come in ``blocks`` equal runs; in run b ``r =
+    sigmoid(A_b u_b + a_b)`` and ``i = sigmoid(B_b u_b + b_b)`` with square matrices ``[out, in]``.  Then ``log a
+    = -rate_scale * r * softplus(lam)``, ``S_t = a S_(t-1) + sqrt(1 - a^2) i u`` (from ``S = 0``, the first
+    token like every other), and the output projection reads ``S * y``.  Everything behind the convolution
+    is fp32; the state row holds S and then the convolution's last ``taps - 1`` inputs."""
+
+    graph_safe = True
+
+    def __init__(self, prefix: str, *, hidden_size: int, width: int, blocks: int, conv_taps: int, rate_scale: float = 8.0,
+                 tensor_names: Optional[Dict[str, str]] = None):
+        """``tensor_names`` maps ``y x y_bias x_bias conv conv_bias a i a_bias i_bias lam o`` to names behind ``prefix``."""
+        super().__init__(prefix)
+        self.hidden_size, self.width, self.blocks, self.conv_taps = int(hidden_size), int(width), int(blocks), int(conv_taps)
+        if self.blocks <= 0 or self.width % self.blocks:
+            raise ValueError(f"{prefix}: {width} channels do not come in {blocks} equal runs")
+        if not 1 <= self.conv_taps <= 17:
+            raise ValueError(f"{prefix}: a convolution of {conv_taps} taps (1..17 are built)")
+        self.rate_scale = float(rate_scale)
+        self.inner_width = self.width
+        self.names = _names(dict(y="y", x="x", y_bias="y.b", x_bias="x.b", conv="conv", conv_bias="conv.b", a="ra", i="ri",
+                                 a_bias="ra.b", i_bias="ri.b", lam="lam", o="o"), tensor_names, prefix)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        n, W, C, B = self.names, self.hidden_size, self.width, self.blocks
+        bs = C // B
+        vec = dict(init="normal", role="vector")
+        return {n["y"]: TensorSpec((C, W)), n["x"]: TensorSpec((C, W)), n["y_bias"]: TensorSpec((C,), **vec),
+                n["x_bias"]: TensorSpec((C,), **vec), n["conv"]: TensorSpec((C, self.conv_taps), init="norm", role="vector"),
+                n["conv_bias"]: TensorSpec((C,), **vec), n["a"]: TensorSpec((B, bs, bs)), n["i"]: TensorSpec((B, bs, bs)),
+                n["a_bias"]: TensorSpec((B, bs), **vec), n["i_bias"]: TensorSpec((B, bs), **vec),
+                n["lam"]: TensorSpec((C,), init="norm", role="vector"), n["o"]: TensorSpec((W, C))}
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        t = {key: tensors[name] for key, name in self.names.items()}
+        self._w_in = torch.cat([t["y"], t["x"]], dim=0).contiguous()
+        self._w_out = t["o"]
+        self.y_off, self.x_off = 0, self.width
+        self.y_bias, self.x_bias = t["y_bias"].float().contiguous(), t["x_bias"].float().contiguous()
+        self.conv_weight, self.conv_bias = t["conv"].float().contiguous(), t["conv_bias"].float().contiguous()
+        self.w_a, self.w_i = t["a"].contiguous(), t["i"].contiguous()
+        self.a_bias, self.i_bias = t["a_bias"].float().reshape(-1).contiguous(), t["i_bias"].float().reshape(-1).contiguous()
+        # the decay's rate per channel, rate_scale * softplus(lam): a constant of the weights, formed once in 32-bit
+        self.rate = (self.rate_scale * torch.nn.functional.softplus(t["lam"].float())).contiguous()
+        self.load_projections()
+
+    def input_weight(self) -> torch.Tensor:
+        return self._w_in
+
+    def output_weight(self) -> torch.Tensor:
+        return self._w_out
+
+    def state_elements(self) -> int:
+        return self.width * self.conv_taps          # S, then taps - 1 inputs per channel
+
+    def activation_elements(self) -> int:
+        return 2 * self.width + 3 * 2 * self.width + self.width + self.hidden_size
+
+    def forward_inner(self, y, col0, ctx: MixerContext, state_off, out, out_col0, mul) -> None:
+        batch, T = ctx.batch, y.shape[0]
+        u = torch.empty((T, self.width), dtype=torch.float32, device=y.device)
+        K.causal_conv_act(y, col0 + self.x_off, self.conv_weight, u, ctx.state, state_off + self.width, batch.entry_q_start,
+                          batch.entry_seat, batch.max_q_len, in_bias=self.x_bias, out_bias=self.conv_bias, activation=None)
+        a, b = torch.empty_like(u), torch.empty_like(u)
+        K.block_gates(u, self.w_a, self.w_i, self.a_bias, self.i_bias, self.rate, a, b)
+        K.linear_scan_gate(a, b, y, col0 + self.y_off, self.y_bias, out, out_col0, ctx.state, state_off,
+                           batch.entry_q_start, batch.entry_seat, mul)

@@ -63,6 +63,13 @@ def plain_frequencies_f64(rot_dim: int, theta: float) -> np.ndarray:
     return np.power(np.float64(theta), -2.0 * i / np.float64(rot_dim))
 
 
+def linear_frequencies_f64(rot_dim: int, theta: float, *, factor: float) -> np.ndarray:
+    """Linear scaling (position interpolation): every plain frequency divided by ``factor``; float64."""
+    if not factor > 0:
+        raise ValueError(f"linear rotary scaling: factor {factor} must be positive")
+    return plain_frequencies_f64(rot_dim, theta) / np.float64(factor)
+
+
 def yarn_frequencies(rot_dim: int, theta: float, *, factor: float, original: float, fast: float,
                      slow: float) -> np.ndarray:
     """YaRN: pair i keeps its plain frequency ``f_i`` where it turns fast and takes ``f_i / factor``
@@ -94,6 +101,7 @@ ROTARY_FREQUENCIES.register("plain", plain_frequencies, replace=True)
 ROTARY_FREQUENCIES.register("llama3", llama3_frequencies, replace=True)
 ROTARY_FREQUENCIES.register("plain_f64", plain_frequencies_f64, replace=True)
 ROTARY_FREQUENCIES.register("yarn", yarn_frequencies, replace=True)
+ROTARY_FREQUENCIES.register("linear_f64", linear_frequencies_f64, replace=True)
 
 
 def rotary_inv_freq(rot_dim: int, theta: float, scaling: Optional[dict]) -> np.ndarray:

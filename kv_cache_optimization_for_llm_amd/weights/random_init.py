@@ -1,7 +1,8 @@
 """Random-weights mode: writes a model folder (``config.json`` + ``model.safetensors``) from a
 configuration and a seed.
 
-Matrices are N(0, 0.02), norm weights 1 + U(-0.1, 0.1).  With a ``gain`` a matrix ``[out, in]``
+Matrices are N(0, 0.02), norm weights 1 + U(-0.1, 0.1), matrices that mix copies of the stream the identity
++ U(-0.1, 0.1).  With a ``gain`` a matrix ``[out, in]``
 is N(0, gain / sqrt(in)) instead: its products of unit-size inputs are of size ``gain`` at any
 width, so attention scores spread and a tied model's best next token is not its input token -
 what tests of generation need from random weights.  Each tensor's generator is seeded from
@@ -42,6 +43,8 @@ def random_tensor(name: str, spec: TensorSpec, seed: int, dtype: torch.dtype,
         t = 1.0 + (torch.rand(spec.shape, generator=g, dtype=torch.float32) * 0.2 - 0.1)
     elif spec.init == "zeros":
         t = torch.zeros(spec.shape, dtype=torch.float32)
+    elif spec.init == "eye":            # a square matrix near the identity
+        t = torch.eye(spec.shape[0], spec.shape[1]) + (torch.rand(spec.shape, generator=g, dtype=torch.float32) * 0.2 - 0.1)
     else:
         raise ValueError(f"tensor {name!r}: unknown init rule {spec.init!r}")
     return t.to(dtype)
@@ -68,6 +71,9 @@ def random_tensors_on_device(specs: Mapping[str, TensorSpec], seed: int, dtype: 
         elif spec.init == "norm":
             t = torch.empty(spec.shape, dtype=torch.float32, device=device).uniform_(0.9, 1.1, generator=g)
             out[name] = t.to(dtype)
+        elif spec.init == "eye":
+            t = torch.empty(spec.shape, dtype=torch.float32, device=device).uniform_(-0.1, 0.1, generator=g)
+            out[name] = (t + torch.eye(spec.shape[0], spec.shape[1], device=device)).to(dtype)
         else:
             out[name] = torch.zeros(spec.shape, dtype=dtype, device=device)
     return out
