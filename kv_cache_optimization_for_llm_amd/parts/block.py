@@ -166,6 +166,8 @@ class HyperConnection(Part):
     weights ``out`` [S] (``x_t <- sum_s mix[s, t] x_s + mult * out[t] * y``).  ``learned=False``: no tensors,
     all of them 1 - with one copy that is the plain residual sum."""
 
+    graph_safe = True
+
     def __init__(self, prefix: str, *, streams: int, learned: bool = True):
         super().__init__(prefix)
         self.streams, self.learned = int(streams), bool(learned)

@@ -20,6 +20,13 @@ from typing import Dict, List, Optional
 import torch
 
 F = torch.float64
+# what a 16-bit engine rounds on its way (projections' results, what the output projections read, the
+# experts' middles): the identity, except while ``forward(rounded=...)`` estimates what rounding does
+_r = lambda t: t  # noqa: E731
+
+
+def to_f64(state: Dict[str, torch.Tensor]) -> Dict[str, torch.Tensor]:
+    return {k: (v.to(F) if v.is_floating_point() else v) for k, v in state.items()}
 
 
 def load_model_dir(path: str):
@@ -67,9 +74,9 @@ def attention(h, Wt, p, m, eps, window: Optional[int]):
     window and a sink per head.  ``h`` [T, width], ``p`` the tensors' prefix, ``m`` the sizes."""
     T = h.shape[0]
     H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = (h @ Wt[p + "q"].T).view(T, H, d)
-    k = (h @ Wt[p + "k"].T).view(T, G, d)
-    v = (h @ Wt[p + "v"].T).view(T, G, dv)
+    q = _r(h @ Wt[p + "q"].T).view(T, H, d)
+    k = _r(h @ Wt[p + "k"].T).view(T, G, d)
+    v = _r(h @ Wt[p + "v"].T).view(T, G, dv)
     q = rms(q, eps) * Wt[p + "q.norm"]
     k = rms(k, eps) * Wt[p + "k.norm"]
     rot = m.get("rot")
@@ -78,6 +85,7 @@ def attention(h, Wt, p, m, eps, window: Optional[int]):
         factor = float((rot.get("scaling") or {}).get("factor", 1.0))
         q = rotate(q, pos, int(rot["dims"]), float(rot["base"]), factor)
         k = rotate(k, pos, int(rot["dims"]), float(rot["base"]), factor)
+    q, k = _r(q), _r(k)
     out = torch.zeros(T, H, dv, dtype=F)
     i = torch.arange(T)[:, None]
     j = torch.arange(T)[None, :]
@@ -93,16 +101,16 @@ def attention(h, Wt, p, m, eps, window: Optional[int]):
         e = torch.exp(s - top)
         den = e.sum(-1, keepdim=True) + torch.exp(sink - top)
         out[:, head] = (e / den) @ v[:, g]
-    return out.reshape(T, H * dv) @ Wt[p + "o"].T
+    return _r(out.reshape(T, H * dv)) @ Wt[p + "o"].T
 
 
 # ---------------------------------------------------------------- matrix memory
 def matrix_memory(h, Wt, p, m, eps):
     T = h.shape[0]
     H, d, dv, cap = m["heads"], m["dim"], m["vdim"], float(m["gate_cap"])
-    q = (h @ Wt[p + "q"].T).view(T, H, d) * d ** -0.5
-    k = (h @ Wt[p + "k"].T).view(T, H, d)
-    v = (h @ Wt[p + "v"].T).view(T, H, dv)
+    q = _r(h @ Wt[p + "q"].T).view(T, H, d) * d ** -0.5
+    k = _r(h @ Wt[p + "k"].T).view(T, H, d)
+    v = _r(h @ Wt[p + "v"].T).view(T, H, dv)
     gi = cap * torch.tanh((h @ Wt[p + "i"].T + Wt[p + "i.b"]) / cap)
     gf = torch.nn.functional.logsigmoid(cap * torch.tanh((h @ Wt[p + "f"].T + Wt[p + "f.b"]) / cap))
     S = torch.zeros(H, d, dv, dtype=F)
@@ -119,16 +127,16 @@ def matrix_memory(h, Wt, p, m, eps):
         den = torch.maximum((n * q[t]).sum(-1).abs(), torch.exp(-mx)) + 1e-6
         o[t] = num / den[:, None]
     o = rms(o, eps).reshape(T, H * dv) * Wt[p + "norm"]
-    o = o * torch.sigmoid(h @ Wt[p + "g"].T)
-    return o @ Wt[p + "o"].T
+    o = o * torch.sigmoid(_r(h @ Wt[p + "g"].T))
+    return _r(o) @ Wt[p + "o"].T
 
 
 # ---------------------------------------------------------------- real-gated linear recurrent unit
 def rglru(h, Wt, p, m):
     T = h.shape[0]
     width, blocks, taps = m["width"], m["blocks"], m["conv"]
-    y = gelu_tanh(h @ Wt[p + "y"].T + Wt[p + "y.b"])
-    x = h @ Wt[p + "x"].T + Wt[p + "x.b"]
+    y = gelu_tanh(_r(h @ Wt[p + "y"].T) + Wt[p + "y.b"])
+    x = _r(h @ Wt[p + "x"].T) + Wt[p + "x.b"]
     conv = Wt[p + "conv"]                                   # [channels, taps], the last column is the current token's
     padded = torch.cat([torch.zeros(taps - 1, width, dtype=F), x], dim=0)
     u = torch.zeros(T, width, dtype=F)
@@ -146,17 +154,17 @@ def rglru(h, Wt, p, m):
     for t in range(T):
         S = a[t] * S + torch.sqrt(1.0 - a[t] ** 2) * g[t] * u[t]
         out[t] = S
-    return (out * y) @ Wt[p + "o"].T
+    return _r(out * y) @ Wt[p + "o"].T
 
 
 # ---------------------------------------------------------------- feed-forwards
 def clamped_expert(h, gate, up, down, limit):
     g = torch.clamp(h @ gate.T, max=limit)
     u = torch.clamp(h @ up.T, -limit, limit)
-    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ down.T
+    return _r(g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ down.T
 
 
-def route(h, Wt, p, mlp, forced: Optional[torch.Tensor] = None):
+def route(h, Wt, p, mlp, forced: Optional[torch.Tensor] = None, margins: Optional[list] = None):
     """(chosen experts [T, top], weights [T, top], choice scores [T, experts] with the left-out groups
     at -inf).  ``forced``: experts to take instead of the router's own choice (the weights follow)."""
     r = mlp["router"]
@@ -172,14 +180,25 @@ def route(h, Wt, p, mlp, forced: Optional[torch.Tensor] = None):
         allowed = torch.zeros(h.shape[0], cnt, dtype=torch.bool)
         allowed.scatter_(1, best, True)
         choice = choice.masked_fill(~allowed[:, :, None].expand(-1, -1, per).reshape(-1, E), -math.inf)
-    idx = choice.topk(top, dim=-1).indices if forced is None else forced.long()
+    best = choice.topk(min(top + 1, E), dim=-1)
+    own = best.indices[:, :top]
+    if margins is not None:
+        # how clear the choice was: the gap between the last expert taken and the first one left out, and -
+        # with groups - between the last group kept and the first one dropped
+        gap = (best.values[:, top - 1] - best.values[:, top]) if E > top else torch.full((h.shape[0],), math.inf, dtype=F)
+        gap = torch.where(torch.isfinite(gap), gap, torch.full_like(gap, math.inf))
+        if groups and int(groups["keep"]) < int(groups["count"]):
+            g2 = gs.topk(int(groups["keep"]) + 1, dim=-1).values
+            gap = torch.minimum(gap, g2[:, -2] - g2[:, -1])
+        margins.append((own, gap))
+    idx = own if forced is None else forced.long()
     w = s.gather(1, idx)
     w = w / (w.sum(-1, keepdim=True) + 1e-20) * float(r.get("scale", 1.0))
     return idx, w, choice
 
 
-def mixture(h, Wt, p, mlp, forced: Optional[torch.Tensor] = None):
-    idx, w, _ = route(h, Wt, p, mlp, forced)
+def mixture(h, Wt, p, mlp, forced: Optional[torch.Tensor] = None, margins: Optional[list] = None):
+    idx, w, _ = route(h, Wt, p, mlp, forced, margins)
     limit = float(mlp["expert"]["limit"])
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
@@ -189,13 +208,13 @@ def mixture(h, Wt, p, mlp, forced: Optional[torch.Tensor] = None):
                                                Wt[f"{p}e{e}.down"], limit)[0]
     shared = mlp.get("shared")
     if shared:
-        y = clamped_expert(h, Wt[p + "shared.gate"], Wt[p + "shared.up"], Wt[p + "shared.down"], float(shared["limit"]))
+        y = _r(clamped_expert(h, Wt[p + "shared.gate"], Wt[p + "shared.up"], Wt[p + "shared.down"], float(shared["limit"])))
         out = out + y * torch.sigmoid(h @ Wt[p + "shared.sg"].T)
     return out
 
 
 def dense(h, Wt, p):
-    return gelu_tanh(h @ Wt[p + "up"].T) @ Wt[p + "down"].T
+    return _r(gelu_tanh(_r(h @ Wt[p + "up"].T))) @ Wt[p + "down"].T
 
 
 # ---------------------------------------------------------------- the model
@@ -220,16 +239,29 @@ def mixer(cfg, Wt, i, h):
     return float(m["left_scale"]) * left + float(m["right_scale"]) * right
 
 
-def feed_forward(cfg, Wt, i, h, forced=None):
+def feed_forward(cfg, Wt, i, h, forced=None, margins=None):
     mlp = cfg["layers"][i]["mlp"]
     if mlp["kind"] == "dense":
         return dense(h, Wt, f"l{i}.mlp.")
-    return mixture(h, Wt, f"l{i}.mlp.", mlp, forced)
+    return mixture(h, Wt, f"l{i}.mlp.", mlp, forced, margins)
 
 
-def forward(cfg, Wt: Dict[str, torch.Tensor], tokens, forced: Optional[dict] = None, layers_out: Optional[list] = None):
+def forward(cfg, Wt: Dict[str, torch.Tensor], tokens, forced: Optional[dict] = None, layers_out: Optional[list] = None,
+            margins: Optional[dict] = None, rounded=None):
     """Logits [T, vocab] of a whole sequence.  ``forced``: {run index: experts [T, top]} to take in
-    place of the routers' own choices; ``layers_out`` receives the stream after every layer run."""
+    place of the routers' own choices; ``layers_out`` receives the stream after every layer run;
+    ``margins`` receives {run index: (the router's own choice, how clear it was)}; ``rounded`` is
+    applied to every branch's input and output (what a 16-bit engine rounds there)."""
+    global _r
+    rounded = rounded or (lambda t: t)
+    _r = rounded
+    try:
+        return _forward(cfg, Wt, tokens, forced, layers_out, margins, rounded)
+    finally:
+        _r = lambda t: t  # noqa: E731
+
+
+def _forward(cfg, Wt, tokens, forced, layers_out, margins, rounded):
     eps, mult = float(cfg["norm"]["eps"]), float(cfg.get("residual_mult", 1.0))
     S = cfg.get("streams")
     x = Wt["embed"][torch.as_tensor(tokens, dtype=torch.long)]
@@ -240,22 +272,25 @@ def forward(cfg, Wt: Dict[str, torch.Tensor], tokens, forced: Optional[dict] = N
         p = f"l{i}."
         w, b = Wt[f"{p}norm{q}"], Wt[f"{p}norm{q}.b"]
         if xs is None:
-            x = x + mult * fn(layer_norm(x, w, b, eps))
+            x = x + mult * rounded(fn(rounded(layer_norm(x, w, b, eps))))
             return
         u = sum(Wt[f"{p}hc{q}.in"][s] * xs[s] for s in range(len(xs)))
-        y = fn(layer_norm(u, w, b, eps))
+        y = rounded(fn(rounded(layer_norm(u, w, b, eps))))
         mix, out = Wt[f"{p}hc{q}.mix"], Wt[f"{p}hc{q}.out"]
         xs = [sum(mix[s, t] * xs[s] for s in range(len(xs))) + mult * out[t] * y for t in range(len(xs))]
 
     for run, i in enumerate(run_order(cfg)):
         sublayer(1, i, lambda h: mixer(cfg, Wt, i, h))
         if cfg["layers"][i].get("mlp") is not None:
-            sublayer(2, i, lambda h: feed_forward(cfg, Wt, i, h, None if forced is None else forced.get(run)))
+            seen = [] if margins is not None else None
+            sublayer(2, i, lambda h: feed_forward(cfg, Wt, i, h, None if forced is None else forced.get(run), seen))
+            if seen:
+                margins[run] = seen[0]
         if layers_out is not None:
             layers_out.append(x.clone() if xs is None else sum(xs))
     if xs is not None:
         x = sum(xs)
-    return layer_norm(x, Wt["final.norm"], Wt["final.norm.b"], eps) @ Wt["head"].T
+    return rounded(layer_norm(x, Wt["final.norm"], Wt["final.norm.b"], eps)) @ Wt["head"].T
 
 
 def generate(cfg, Wt, prompt, new_tokens: int) -> List[int]:

@@ -1,0 +1,291 @@
+"""The kernels that came with the Bonusun decoder, each alone against a few lines of plain PyTorch (float64):
+the step between two branches over several copies of the stream, the router that chooses inside groups,
+the clamped gated activation, the activation with a bias, head norms before the rotation, the convolution
+with biases, the real-gated recurrence (gates and scan) and the matrix memory - the recurrences cut into
+steps of 1, 2, 17, ... tokens over seats that are used again."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from kv_cache_optimization_for_llm_amd.ops import kernels as K
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+F64 = torch.float64
+
+
+def rnd(shape, seed, std=1.0, mean=0.0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * std + mean).to(dtype).to(DEV)
+
+
+def close(got, want, tol, what=""):
+    got, want = got.detach().double().cpu(), want.detach().double().cpu()
+    err = (got - want).abs().max().item()
+    assert err <= tol * max(1.0, want.abs().max().item()), f"{what}: off by {err:.3g}"
+
+
+# ---------------------------------------------------------------- copies of the stream
+@pytest.mark.parametrize("S, width", [(1, 40), (2, 256), (3, 96), (4, 1000), (8, 64)])
+@pytest.mark.parametrize("ydtype", [torch.float32, torch.bfloat16])
+def test_the_step_between_two_branches(S, width, ydtype, gpu):
+    T = 7
+    x = rnd((T, S * width), 1, 2.0)
+    y = rnd((T, width), 2, dtype=ydtype)
+    mix, out_w, in_w = rnd((S, S), 3, 0.5), rnd((S,), 4), rnd((S,), 5)
+    nw, nb = rnd((width,), 6, 0.3, 1.0, ydtype), rnd((width,), 7, 0.3, dtype=ydtype)
+    mult, eps = 0.7, 1e-3
+    xs = x.double().view(T, S, width)
+    new = torch.einsum("st,bsw->btw", mix.double(), xs) + mult * out_w.double()[None, :, None] * y.double()[:, None, :]
+    u = (in_w.double()[None, :, None] * new).sum(1)
+    want = (u - u.mean(-1, keepdim=True)) / torch.sqrt(u.var(-1, unbiased=False, keepdim=True) + eps) * nw.double() + nb.double()
+    # enter and read out in one launch
+    x1, out = x.clone(), torch.empty((T, width), dtype=ydtype, device=DEV)
+    K.hyper_step(x1, S, y=y, mix=mix, out_w=out_w, mult=mult, in_w=in_w, norm_weight=nw, norm_bias=nb, eps=eps, out=out)
+    close(x1.view(T, S, width), new, 1e-5, "copies")
+    close(out, want, 1e-5 if ydtype == torch.float32 else 1e-2, "read-out")
+    # enter alone, then read out alone (and without a bias): the same copies, the same rows
+    x2 = x.clone()
+    K.hyper_step(x2, S, y=y, mix=mix, out_w=out_w, mult=mult)
+    assert torch.equal(x1, x2)
+    out2 = torch.empty_like(out)
+    K.hyper_step(x2, S, in_w=in_w, norm_weight=nw, norm_bias=None, eps=eps, out=out2)
+    close(out2, want - nb.double(), 1e-5 if ydtype == torch.float32 else 2e-2, "without bias")
+    assert torch.equal(x1, x2), "reading out changes nothing"
+    # gathered rows: nothing is written back
+    idx = torch.tensor([5, 0, 5], dtype=torch.int32, device=DEV)
+    x3, out3 = x.clone(), torch.empty((3, width), dtype=ydtype, device=DEV)
+    K.hyper_step(x3, S, y=y, mix=mix, out_w=out_w, mult=mult, in_w=in_w, norm_weight=nw, norm_bias=nb, eps=eps, out=out3, row_idx=idx)
+    assert torch.equal(x3, x) and torch.equal(out3, out[idx.long()])
+
+
+def test_every_copy_starts_as_the_embedding_output(gpu):
+    first = rnd((5, 24), 1)
+    x = torch.empty((5, 3 * 24), device=DEV)
+    K.hyper_fill(x, first, 3)
+    assert torch.equal(x.view(5, 3, 24), first[:, None, :].expand(5, 3, 24))
+
+
+# ---------------------------------------------------------------- activations
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_clamped_gated_activation_and_activation_with_bias(dtype, gpu):
+    gu = rnd((9, 2 * 40), 1, 2.0, dtype=dtype)
+    out = torch.empty((9, 40), dtype=dtype, device=DEV)
+    K.act_mul(gu, out, "swish_clamped", 1.3)
+    g, u = gu.double()[:, :40].clamp(max=1.3), gu.double()[:, 40:].clamp(-1.3, 1.3)
+    close(out, g * torch.sigmoid(1.702 * g) * (u + 1), 1e-6 if dtype == torch.float32 else 1e-2)
+    x, b = rnd((9, 52), 2, 2.0, dtype=dtype), rnd((52,), 3)
+    z = x.double() + b.double()
+    want = 0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3)))
+    close(K.bias_act(x, torch.empty_like(x), "gelu_tanh", b), want, 1e-6 if dtype == torch.float32 else 1e-2)
+    close(K.bias_act(x, x.clone(), "relu"), x.double().clamp(min=0), 1e-6)
+
+
+# ---------------------------------------------------------------- router
+def plain_route(logits, corr, top, groups, keep, scale, eps=1e-20):
+    s = torch.sigmoid(logits.double())
+    ch = s + corr.double()
+    T, E = s.shape
+    idx, wgt = [], []
+    for t in range(T):
+        c = ch[t].clone()
+        if groups > 1:
+            per = E // groups
+            score = [sorted(c[g * per:(g + 1) * per].tolist(), reverse=True)[:2] for g in range(groups)]
+            order = sorted(range(groups), key=lambda g: (-sum(score[g]), g))[:keep]
+            for g in range(groups):
+                if g not in order:
+                    c[g * per:(g + 1) * per] = -math.inf
+        pick = sorted(range(E), key=lambda e: (-c[e].item(), e))[:top]
+        w = s[t, pick]
+        idx.append(pick)
+        wgt.append(w / (w.sum() + eps) * scale)
+    return torch.tensor(idx), torch.stack(wgt)
+
+
+@pytest.mark.parametrize("E, top, groups, keep", [(12, 4, 4, 3), (6, 2, 3, 2), (4, 1, 4, 2), (8, 8, 1, 1), (64, 6, 8, 2),
+                                                  (130, 5, 1, 1), (9, 3, 3, 1), (16, 4, 2, 2)])
+def test_the_router_chooses_inside_the_best_groups(E, top, groups, keep, gpu):
+    T = 50
+    logits = rnd((T, E), E, 2.0)
+    corr = rnd((E,), E + 1, 0.5, -1.5)        # choice scores below zero: a group left out counts as -inf, not as 0
+    idx = torch.empty((T, top), dtype=torch.int32, device=DEV)
+    wgt = torch.empty((T, top), dtype=torch.float32, device=DEV)
+    K.moe_route(logits, corr, top, idx, wgt, renormalise=True, scores="sigmoid", groups=groups, keep_groups=keep,
+                group_top=2, weight_scale=1.5, sum_eps=1e-20)
+    want_idx, want_w = plain_route(logits.cpu(), corr.cpu(), top, groups, keep, 1.5)
+    assert torch.equal(idx.cpu().long(), want_idx)
+    close(wgt, want_w, 1e-6)
+
+
+# ---------------------------------------------------------------- head norms before the rotation
+@pytest.mark.parametrize("d, rot", [(16, 8), (32, 32), (24, 0), (64, 16)])
+def test_heads_are_normed_and_then_rotated(d, rot, gpu):
+    T, H = 6, 3
+    q = rnd((T, H * d), 1)
+    pos = torch.tensor([0, 1, 5, 17, 40, 63], dtype=torch.int32, device=DEV)
+    wq = rnd((d,), 2, 0.3, 1.0)
+    cos = sin = None
+    x = q.double().view(T, H, d)
+    x = x / torch.sqrt((x * x).mean(-1, keepdim=True) + 0.01) * wq.double()
+    if rot:
+        f = torch.tensor([100.0 ** (-2 * i / rot) for i in range(rot // 2)], dtype=F64)
+        ang = torch.arange(64, dtype=F64)[:, None] * f
+        cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
+        a = ang[pos.cpu().long()][:, None, :].to(DEV)
+        u, v = x[..., :rot // 2], x[..., rot // 2:rot]
+        x = torch.cat([u * torch.cos(a) - v * torch.sin(a), v * torch.cos(a) + u * torch.sin(a), x[..., rot:]], -1)
+    K.qk_encode_cache(q, pos, H, 0, d, d, cos, sin, False, 0.01, None, None, None, q_weight=wq, norm_first=True)
+    close(q.view(T, H, d), x, 1e-5)
+
+
+# ---------------------------------------------------------------- entries over seats
+def entries(lengths, seats):
+    starts = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    return torch.from_numpy(starts).to(DEV), torch.tensor(seats, dtype=torch.int32, device=DEV)
+
+
+def walk(total_lengths, cuts):
+    """Steps that take every request's tokens in portions of ``cuts`` (cycled): yields (lo, hi) per request."""
+    at = [0] * len(total_lengths)
+    k = 0
+    while any(a < n for a, n in zip(at, total_lengths)):
+        step = []
+        for r, n in enumerate(total_lengths):
+            take = min(cuts[k % len(cuts)], n - at[r])
+            step.append((at[r], at[r] + take))
+            at[r] += take
+            k += 1
+        yield step
+
+
+@pytest.mark.parametrize("taps", [1, 2, 4, 17])
+def test_convolution_with_biases_and_no_activation_over_steps(taps, gpu):
+    C, lengths = 20, [37, 5]
+    y = [rnd((n, C + 3), 10 + i) for i, n in enumerate(lengths)]
+    w, ib, ob = rnd((C, taps), 1), rnd((C,), 2), rnd((C,), 3)
+    state = rnd((4, 7 + C * (taps - 1)), 4)
+    state[:, 7:] = 0
+    got = [torch.empty((n, C), device=DEV) for n in lengths]
+    for step in walk(lengths, (1, 2, 17, 3)):
+        rows = torch.cat([y[r][lo:hi] for r, (lo, hi) in enumerate(step)])
+        out = torch.empty((rows.shape[0], C), device=DEV)
+        qs, seat = entries([hi - lo for lo, hi in step], [2, 0])
+        K.causal_conv_act(rows, 3, w, out, state, 7, qs, seat, max(hi - lo for lo, hi in step), in_bias=ib, out_bias=ob,
+                          activation=None)
+        at = 0
+        for r, (lo, hi) in enumerate(step):
+            got[r][lo:hi] = out[at:at + hi - lo]
+            at += hi - lo
+    for r, n in enumerate(lengths):
+        x = torch.cat([torch.zeros((taps - 1, C), dtype=F64, device=DEV), y[r][:, 3:].double() + ib.double()])
+        want = sum(x[j:j + n] * w.double()[:, j] for j in range(taps)) + ob.double()
+        close(got[r], want, 1e-5, f"request {r}")
+
+
+@pytest.mark.parametrize("width, blocks", [(24, 24), (40, 1), (128, 2), (200, 2), (96, 3)])
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
+def test_real_gated_recurrence_over_steps_and_seats_used_again(width, blocks, wdtype, gpu):
+    bs = width // blocks
+    lengths = [300, 1, 45]
+    u = [rnd((n, width), 20 + i) for i, n in enumerate(lengths)]
+    gate = [rnd((n, width + 5), 30 + i, dtype=wdtype) for i, n in enumerate(lengths)]
+    wa, wi = rnd((blocks, bs, bs), 1, 1 / bs ** 0.5, dtype=wdtype), rnd((blocks, bs, bs), 2, 1 / bs ** 0.5, dtype=wdtype)
+    ba, bi, lam, gb = rnd((width,), 3), rnd((width,), 4), rnd((width,), 5, 1.0, -1.0), rnd((width,), 6)
+    rate = (8.0 * torch.nn.functional.softplus(lam)).contiguous()
+    state = rnd((3, 11 + width), 7)          # what an earlier request left in the seats ...
+    seats = [1, 0, 2]
+    got = [torch.empty((n, width), device=DEV) for n in lengths]
+    first = True
+    for step in walk(lengths, (1, 2, 17, 64, 33)):
+        live = [(r, lo, hi) for r, (lo, hi) in enumerate(step) if hi > lo]
+        if first:
+            state[:, 11:] = 0                # ... is gone when a request takes the seat
+            first = False
+        rows_u = torch.cat([u[r][lo:hi] for r, lo, hi in live])
+        rows_g = torch.cat([gate[r][lo:hi] for r, lo, hi in live])
+        a, b = torch.empty_like(rows_u), torch.empty_like(rows_u)
+        K.block_gates(rows_u, wa, wi, ba, bi, rate, a, b)
+        out = torch.zeros((rows_u.shape[0], width + 2), device=DEV)
+        qs, seat = entries([hi - lo for _, lo, hi in live], [seats[r] for r, _, _ in live])
+        K.linear_scan_gate(a, b, rows_g, 5, gb, out, 2, state, 11, qs, seat, 0.5)
+        at = 0
+        for r, lo, hi in live:
+            got[r][lo:hi] = out[at:at + hi - lo, 2:]
+            at += hi - lo
+    for r, n in enumerate(lengths):
+        ub = u[r].double().view(n, blocks, bs)
+        rr = torch.sigmoid(torch.einsum("tbi,boi->tbo", ub, wa.double()).reshape(n, width) + ba.double())
+        ii = torch.sigmoid(torch.einsum("tbi,boi->tbo", ub, wi.double()).reshape(n, width) + bi.double())
+        aa = torch.exp(-8.0 * rr * torch.nn.functional.softplus(lam.double()))
+        S = torch.zeros(width, dtype=F64, device=DEV)
+        z = gate[r][:, 5:].double() + gb.double()
+        act = 0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3)))
+        want = torch.empty((n, width), dtype=F64, device=DEV)
+        for t in range(n):
+            S = aa[t] * S + torch.sqrt(1 - aa[t] ** 2) * ii[t] * u[r][t].double()
+            want[t] = S * act[t] * 0.5
+        close(got[r], want, 2e-5, f"request {r}")
+        close(state[seats[r], 11:], S, 2e-5, f"state of request {r}")
+
+
+@pytest.mark.parametrize("H, d, dv", [(3, 16, 24), (1, 8, 40), (4, 32, 48), (2, 160, 8), (2, 64, 64)])
+@pytest.mark.parametrize("ydtype", [torch.float32, torch.bfloat16])
+def test_matrix_memory_over_steps_and_seats_used_again(H, d, dv, ydtype, gpu):
+    lengths, cap = [70, 2, 33], 5.0
+    cols = 3 + 2 * H * d + H * dv
+    y = [rnd((n, cols), 40 + i, dtype=ydtype) for i, n in enumerate(lengths)]
+    gates = [rnd((n, 2 * H), 50 + i, 2.0, 0.5) for i, n in enumerate(lengths)]
+    n_state = K.matrix_memory_state(H, d, dv)
+    state = rnd((3, 4 + n_state), 8)
+    state[:, 4:] = 0
+    seats = [2, 0, 1]
+    got = [torch.empty((n, H * dv), device=DEV) for n in lengths]
+    for step in walk(lengths, (1, 2, 17, 16, 5)):
+        live = [(r, lo, hi) for r, (lo, hi) in enumerate(step) if hi > lo]
+        rows = torch.cat([y[r][lo:hi] for r, lo, hi in live])
+        g = torch.cat([gates[r][lo:hi] for r, lo, hi in live])
+        out = torch.empty((rows.shape[0], H * dv), device=DEV)
+        qs, seat = entries([hi - lo for _, lo, hi in live], [seats[r] for r, _, _ in live])
+        K.matrix_memory(rows, 3, 3 + H * d, 3 + 2 * H * d, g, cap, d ** -0.5, out, state, 4, qs, seat, H, d, dv)
+        at = 0
+        for r, lo, hi in live:
+            got[r][lo:hi] = out[at:at + hi - lo]
+            at += hi - lo
+    for r, n in enumerate(lengths):
+        yy = y[r].double()
+        q = yy[:, 3:3 + H * d].view(n, H, d) * d ** -0.5
+        k = yy[:, 3 + H * d:3 + 2 * H * d].view(n, H, d)
+        v = yy[:, 3 + 2 * H * d:].view(n, H, dv)
+        gi = cap * torch.tanh(gates[r][:, :H].double() / cap)
+        gf = torch.nn.functional.logsigmoid(cap * torch.tanh(gates[r][:, H:].double() / cap))
+        S = torch.zeros((H, d, dv), dtype=F64, device=DEV)
+        nn = torch.zeros((H, d), dtype=F64, device=DEV)
+        m = torch.zeros(H, dtype=F64, device=DEV)
+        want = torch.empty((n, H, dv), dtype=F64, device=DEV)
+        for t in range(n):
+            new = torch.maximum(gf[t] + m, gi[t])
+            keep, take = torch.exp(gf[t] + m - new), torch.exp(gi[t] - new)
+            S = keep[:, None, None] * S + take[:, None, None] * k[t][:, :, None] * v[t][:, None, :]
+            nn = keep[:, None] * nn + take[:, None] * k[t]
+            m = new
+            den = torch.maximum((nn * q[t]).sum(-1).abs(), torch.exp(-m)) + 1e-6
+            want[t] = torch.einsum("hdv,hd->hv", S, q[t]) / den[:, None]
+        close(got[r], want.view(n, H * dv), 5e-5, f"request {r}")
+        close(state[seats[r], 4:4 + H * d * dv], S.reshape(-1), 5e-5, f"matrix of request {r}")
+
+
+@pytest.mark.parametrize("heads, dv", [(4, 48), (1, 40), (3, 8)])
+def test_head_norm_with_a_weight_of_all_heads_size_and_without_a_gate(heads, dv, gpu):
+    T = 5
+    x, w, gate = rnd((T, heads * dv), 1), rnd((heads * dv,), 2, 0.3, 1.0), rnd((T, heads * dv + 4), 3)
+    out = torch.zeros((T, heads * dv + 6), device=DEV)
+    K.head_norm_gate(x, w, 0.01, gate, 4, out, 6, heads, dv, "sigmoid", 1.1)
+    xs = x.double().view(T, heads, dv)
+    n = (xs / torch.sqrt((xs * xs).mean(-1, keepdim=True) + 0.01)).reshape(T, -1) * w.double()
+    close(out[:, 6:], n * torch.sigmoid(gate[:, 4:].double()) * 1.1, 1e-5)
+    out2 = torch.zeros((T, heads * dv + 6), device=DEV)
+    K.head_norm_gate(x, None, 0.0, None, 0, out2, 6, heads, dv, None, 0.8)
+    close(out2[:, 6:], x.double() * 0.8, 1e-6)
