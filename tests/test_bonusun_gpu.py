@@ -158,16 +158,21 @@ def test_sharp_scores_at_window_edges_sinks_and_far_keys(name, gain, cuts, dtype
     token off it, and decoded one by one; and - in the layers without a window - a key hundreds of positions
     back.  (A: the kernels for values of another size than the keys; C: the bf16 engine's matrix-core kernels.)"""
     cfg = U.CONFIGS[name][0]
+    if dtype == "bfloat16":
+        gain = min(gain, 2.0)          # (in 16 bits a softmax four times as sharp turns rounding into other keys)
+    if name == "A":
+        # (every run of a layer with softmaxes that sharp doubles or triples what rounding did before it: the
+        # looped layers run once here, five layer runs in all)
+        cfg = dict(cfg, loop=dict(cfg["loop"], times=1))
     folder, state = U.write_model(str(tmp_path / "sharp"), cfg, 21, edit=_sharp(cfg, gain))
     reqs = {"e0": U.prompt(cfg, 75, 1), "e1": U.prompt(cfg, 340, 2)}
     eng = engine_for(folder, dtype)
-    # (softmaxes that sharp multiply the rounding of what they read, and A's nine layer runs double a row's
-    # error each: a 32-bit row may be off by 3e-3 - a key wrongly seen or hidden moves it by a hundred times
-    # that - and in bfloat16 the routers behind them see it:
-    # there a router's choice is held to the rows' limits alone in A, nine layer runs deep, and to gaps of
-    # 0.3 in C; in 32-bit no gap is forgiven)
+    # (softmaxes that sharp multiply the rounding of what they read: a 32-bit row may be off by 1e-3 - a key
+    # wrongly seen or hidden moves it by a hundred times that - and in bfloat16 the routers behind them see it:
+    # there a router's choice is held to the rows' limits alone in A and to gaps of 0.3 in C; in 32-bit no gap
+    # is forgiven)
     close = None if dtype == "float32" else (1.0 if name == "A" else 0.3)
-    tol = 3e-3
+    tol = 1e-3
     check(eng, cfg, state, reqs, R.whole(reqs), dtype, "whole", close, tol)
     check(eng, cfg, state, reqs, R.chunked(reqs, cuts), dtype, "cuts at window lengths", close, tol)
     check(eng, cfg, state, {"e0": reqs["e0"]}, R.tail_decoded({"e0": reqs["e0"]}, tail=60), dtype, "decoded over window edges", close, tol)
