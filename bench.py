@@ -15,7 +15,7 @@ tokens, each with its step time, bytes and fraction of the HBM peak, and the ser
 (``kclass_...``; ``--no-kernel-classes`` leaves them out) and, for the serving runs, pages reused,
 preemptions and fragmentation failures.
 
-    python bench.py --design gadopel|radilix|lomodra [--layers 8]
+    python bench.py --design gadopel|radilix|lomodra|bonusun [--layers 8]
 
 is another measurement with a JSON line of its own (the default run above is untouched): prefill
 and decode throughput of a Gadopel model at layer sizes of a served model (random weights), beside
@@ -133,6 +133,30 @@ def lomodra_config(layers: int, vocab: int, width: int = 2048) -> dict:
             "token_side": {"dim": 64}, "layers": [kinds[i % 4](i) for i in range(layers)], "max_positions": 8192}
 
 
+# --design bonusun: layers of width W in runs of four over four copies of the stream - a real-gated linear
+# recurrent unit (W channels in runs of 256, four taps), softmax attention inside a window of 1,024 positions
+# (W / 64 heads of 64 over W / 256 kv heads, normed queries and keys, a sink), such an attention without a
+# window beside a matrix memory (W / 128 heads of 64 x 128), and windowed attention again.  Every layer has 16
+# clamped gated experts of width 3 W / 8 in 4 groups of which 2 are kept, 4 choices a token, and one more
+# expert of that width that every token uses.  Beside it run the closest design, Radilix (mixers side by side,
+# recurrences and routed experts too), and the Llama model, both at the same width.
+def bonusun_config(layers: int, vocab: int, width: int = 2048) -> dict:
+    W = width
+    mlp = {"kind": "moe", "expert": {"ff": 3 * W // 8, "limit": 7.0},
+           "router": {"experts": 16, "top": 4, "groups": {"count": 4, "keep": 2}, "scale": 2.5},
+           "shared": {"ff": 3 * W // 8, "limit": 7.0}}
+    attn = {"heads": W // 64, "kv_heads": W // 256, "dim": 64, "vdim": 64, "scale": 0.125, "rot": {"base": 500000.0, "dims": 64}}
+    kinds = [
+        {"type": "rglru", "mlp": mlp, "mixer": {"width": W, "blocks": W // 256, "conv": 4}},
+        {"type": "attention", "mlp": mlp, "mixer": dict(attn, mask={"size": 1024})},
+        {"type": "parallel", "mlp": mlp, "mixer": {"left": dict(attn), "left_scale": 1.0, "right_scale": 0.5,
+                                                   "right": {"heads": W // 128, "dim": 64, "vdim": 128, "gate_cap": 15.0}}},
+        {"type": "attention", "mlp": mlp, "mixer": dict(attn, mask={"size": 1024})},
+    ]
+    return {"architecture": "Bonusun", "vocab": vocab, "width": W, "norm": {"eps": 1e-6}, "residual_mult": 0.7, "streams": 4,
+            "layers": [kinds[i % 4] for i in range(layers)], "max_positions": 8192}
+
+
 def design_comparison(args) -> int:
     import torch
     from kv_cache_optimization_for_llm_amd.engine.batch import StepEntry
@@ -143,13 +167,15 @@ def design_comparison(args) -> int:
     llama = dict(CONFIG_1B, num_hidden_layers=layers, vocab_size=vocab, tie_word_embeddings=False)
     design, width = args.design, args.width
     if width != 2048:
-        if design not in ("radilix", "lomodra") or width % 512 or not 512 <= width <= 8192:
-            print("--width: a multiple of 512 from 512 to 8192, for --design radilix or lomodra")
+        if design not in ("radilix", "lomodra", "bonusun") or width % 512 or not 512 <= width <= 8192:
+            print("--width: a multiple of 512 from 512 to 8192, for --design radilix, lomodra or bonusun")
             return 2
         llama.update(hidden_size=width, intermediate_size=4 * width, num_attention_heads=width // 64,
                      num_key_value_heads=width // 256)
     if design == "lomodra":
         configs = {design: lomodra_config(layers, vocab, width), "radilix": radilix_config(layers, vocab, width), "llama": llama}
+    elif design == "bonusun":
+        configs = {design: bonusun_config(layers, vocab, width), "radilix": radilix_config(layers, vocab, width), "llama": llama}
     elif design == "radilix":
         configs = {design: radilix_config(layers, vocab, width), "llama": llama}
     else:
@@ -237,10 +263,10 @@ def design_comparison(args) -> int:
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", choices=["gadopel", "radilix", "lomodra"], default=None,
+    ap.add_argument("--design", choices=["gadopel", "radilix", "lomodra", "bonusun"], default=None,
                     help="another measurement (its own JSON line): a model of this design at the layer sizes of a "
                          "served model beside a Llama model of equal size; the default run is left as it is")
-    ap.add_argument("--width", type=int, default=2048, help="--design radilix or lomodra: the models' width (head counts and "
+    ap.add_argument("--width", type=int, default=2048, help="--design radilix, lomodra or bonusun: the models' width (head counts and "
                     "feed-forward sizes scale with it)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)

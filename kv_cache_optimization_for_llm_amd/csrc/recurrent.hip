@@ -794,51 +794,135 @@ extern "C" int kva_head_norm_gate(void *out, int out_dtype, int out_stride, int 
 // S_t = a_t S_(t-1) + sqrt(1 - a_t^2) i_t u_t with log a_t = -rate_c r_t (rate_c = 8 softplus(lam_c), formed
 // once when the weights are loaded) is linear in S, so this kernel forms, for all tokens side by side,
 // a_t and the input b_t = sqrt(1 - a_t^2) i_t u_t, and kva_linear_scan_gate walks the tokens.
-// A workgroup takes 16 tokens x 64 outputs of one run; thread (row, cx) four neighbouring outputs.
-// k ascending: a token's numbers do not depend on the batch.
+// A workgroup takes 64 tokens x 64 outputs of one run, a thread 4 x 4 of them for both matrices (operands
+// through LDS, 16 inputs at a time).  k ascending into one accumulator per output: a token's numbers do not
+// depend on the batch.
+#define BG_BM 64
+#define BG_BN 64
+#define BG_BK 16
 __global__ void __launch_bounds__(256)
 block_gates_kernel(float *__restrict__ a_out, float *__restrict__ b_out, const float *__restrict__ u, int tokens, int width,
                    int bs, const void *__restrict__ wa, const void *__restrict__ wi, int w_dtype,
                    const float *__restrict__ ba, const float *__restrict__ bi, const float *__restrict__ rate) {
-    __shared__ float us[16][33], was[64][33], wis[64][33];
-    const int blk = blockIdx.y, t0 = blockIdx.z * 16, n0 = blockIdx.x * 64;
-    const int row = threadIdx.x / 16, cx = threadIdx.x % 16;
+    __shared__ float Us[BG_BK][BG_BM + 4], Was[BG_BK][BG_BN + 4], Wis[BG_BK][BG_BN + 4];
+    const int blk = blockIdx.y, t0 = blockIdx.z * BG_BM, n0 = blockIdx.x * BG_BN;
+    const int tid = threadIdx.x, tx = tid % 16, ty = tid / 16;
+    const int lrow = tid / 4, lk = (tid % 4) * 4;
     const size_t wbase = (size_t)blk * bs * bs;
-    float ar[4] = {0.f, 0.f, 0.f, 0.f}, ai[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int k0 = 0; k0 < bs; k0 += 32) {
-        __syncthreads();
-        for (int i = threadIdx.x; i < 16 * 32; i += 256) {
-            const int rr = i / 32, kk = k0 + i % 32;
-            us[rr][i % 32] = (t0 + rr < tokens && kk < bs) ? u[(size_t)(t0 + rr) * width + blk * bs + kk] : 0.f;
-        }
-        for (int i = threadIdx.x; i < 64 * 32; i += 256) {
-            const int nn = n0 + i / 32, kk = k0 + i % 32;
-            const bool in = nn < bs && kk < bs;
-            was[i / 32][i % 32] = in ? rec_ld(wa, w_dtype, wbase + (size_t)nn * bs + kk) : 0.f;
-            wis[i / 32][i % 32] = in ? rec_ld(wi, w_dtype, wbase + (size_t)nn * bs + kk) : 0.f;
-        }
-        __syncthreads();
-        for (int kk = 0; kk < 32; ++kk) {
-            const float xv = us[row][kk];
+    float ar[4][4], ai[4][4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                ar[j] += xv * was[4 * cx + j][kk];
-                ai[j] += xv * wis[4 * cx + j][kk];
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) ar[i][j] = ai[i][j] = 0.f;
+    for (int k0 = 0; k0 < bs; k0 += BG_BK) {
+        float xa[4], xr[4], xi[4];
+        const int tok = t0 + lrow, wn = n0 + lrow;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int kk = k0 + lk + e;
+            xa[e] = (tok < tokens && kk < bs) ? u[(size_t)tok * width + blk * bs + kk] : 0.f;
+            const bool in = wn < bs && kk < bs;
+            xr[e] = in ? rec_ld(wa, w_dtype, wbase + (size_t)wn * bs + kk) : 0.f;
+            xi[e] = in ? rec_ld(wi, w_dtype, wbase + (size_t)wn * bs + kk) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            Us[lk + e][lrow] = xa[e];
+            Was[lk + e][lrow] = xr[e];
+            Wis[lk + e][lrow] = xi[e];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < BG_BK; ++kk) {
+            float uv[4], rv[4], iv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                uv[i] = Us[kk][4 * ty + i];
+                rv[i] = Was[kk][4 * tx + i];
+                iv[i] = Wis[kk][4 * tx + i];
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    ar[i][j] += uv[i] * rv[j];
+                    ai[i][j] += uv[i] * iv[j];
+                }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int t = t0 + 4 * ty + i;
+        if (t >= tokens) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + 4 * tx + j;
+            if (n >= bs) continue;
+            const int c = blk * bs + n;
+            const float r = rec_sigmoid(ar[i][j] + ba[c]), g = rec_sigmoid(ai[i][j] + bi[c]);
+            const float log_a = -rate[c] * r;
+            const size_t at = (size_t)t * width + c;
+            a_out[at] = expf(log_a);
+            b_out[at] = sqrtf(-expm1f(2.f * log_a)) * g * u[at];          // sqrt(1 - a^2) without the cancellation near a = 1
+        }
+    }
+}
+
+// Few tokens (decoding): a workgroup takes a token and 64 channels; the token's inputs go to LDS once, a
+// wavefront takes 16 channels, four at a time with 16 lanes a channel: the lanes stride over the run's inputs
+// (bf16 matrices with runs that are multiples of 8: 16 bytes a lane and load), all loads of the four rounds
+// are independent of each other, and the 16 lanes add up by rotations inside their row of lanes.
+__global__ void __launch_bounds__(256)
+block_gates_rows_kernel(float *__restrict__ a_out, float *__restrict__ b_out, const float *__restrict__ u, int width, int bs,
+                        const void *__restrict__ wa, const void *__restrict__ wi, int w_dtype,
+                        const float *__restrict__ ba, const float *__restrict__ bi, const float *__restrict__ rate) {
+    extern __shared__ float us[];
+    const size_t t = blockIdx.x;
+    const int c_lo = blockIdx.y * 64;
+    const int lane = threadIdx.x % KVA_WAVE, wave = threadIdx.x / KVA_WAVE, r16 = lane % 16, sub = lane / 16;
+    // (the inputs of the runs this workgroup's channels lie in)
+    const int k_lo = (c_lo / bs) * bs, k_hi = min(width, ((min(c_lo + 64, width) - 1) / bs + 1) * bs);
+    for (int k = k_lo + threadIdx.x; k < k_hi; k += blockDim.x) us[k - k_lo] = u[t * width + k];
+    __syncthreads();
+    const bool vec = w_dtype == KVA_BF16 && bs % 8 == 0;
+    float ar[4], ai[4];
+#pragma unroll
+    for (int round = 0; round < 4; ++round) {
+        const int c = c_lo + 16 * wave + 4 * round + sub;
+        ar[round] = ai[round] = 0.f;
+        if (c >= width) continue;
+        const int blk = c / bs;
+        const size_t wrow = (size_t)blk * bs * bs + (size_t)(c - blk * bs) * bs;
+        const float *xs = us + (blk * bs - k_lo);
+        if (vec) {
+            for (int k = 8 * r16; k < bs; k += 128) {
+                const uint4 va = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(wa) + wrow + k);
+                const uint4 vi = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(wi) + wrow + k);
+                const uint32_t pa[4] = {va.x, va.y, va.z, va.w}, pi[4] = {vi.x, vi.y, vi.z, vi.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    ar[round] += xs[k + 2 * e] * __uint_as_float(pa[e] << 16) + xs[k + 2 * e + 1] * __uint_as_float(pa[e] & 0xffff0000u);
+                    ai[round] += xs[k + 2 * e] * __uint_as_float(pi[e] << 16) + xs[k + 2 * e + 1] * __uint_as_float(pi[e] & 0xffff0000u);
+                }
+            }
+        } else {
+            for (int k = r16; k < bs; k += 16) {
+                ar[round] += xs[k] * rec_ld(wa, w_dtype, wrow + k);
+                ai[round] += xs[k] * rec_ld(wi, w_dtype, wrow + k);
             }
         }
     }
-    const int t = t0 + row;
-    if (t >= tokens) return;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int n = n0 + 4 * cx + j;
-        if (n >= bs) continue;
-        const int c = blk * bs + n;
-        const float r = rec_sigmoid(ar[j] + ba[c]), g = rec_sigmoid(ai[j] + bi[c]);
-        const float log_a = -rate[c] * r;
-        const size_t at = (size_t)t * width + c;
-        a_out[at] = expf(log_a);
-        b_out[at] = sqrtf(-expm1f(2.f * log_a)) * g * u[at];          // sqrt(1 - a^2) without the cancellation near a = 1
+    for (int round = 0; round < 4; ++round) {
+        const int c = c_lo + 16 * wave + 4 * round + sub;
+        const float sr = row16_sum(ar[round]), si = row16_sum(ai[round]);
+        if (r16 == 0 && c < width) {
+            const float r = rec_sigmoid(sr + ba[c]), g = rec_sigmoid(si + bi[c]);
+            const float log_a = -rate[c] * r;
+            a_out[t * width + c] = expf(log_a);
+            b_out[t * width + c] = sqrtf(-expm1f(2.f * log_a)) * g * us[c - k_lo];
+        }
     }
 }
 
@@ -850,8 +934,18 @@ extern "C" int kva_block_gates(float *a_out, float *b_out, const float *u, int t
     KVA_REQUIRE(w_dtype == KVA_BF16 || w_dtype == KVA_F32, "block_gates: unsupported dtype");
     if (tokens == 0) return KVA_OK;
     const int bs = width / blocks;
-    KVA_REQUIRE(blocks <= 65535 && (tokens + 15) / 16 <= 65535, "block_gates: too many runs or tokens for one launch");
-    hipLaunchKernelGGL(block_gates_kernel, dim3((bs + 63) / 64, blocks, (tokens + 15) / 16), dim3(256), 0, stream, a_out, b_out,
+    if (tokens <= 32 && (width + 63) / 64 <= 65535) {
+        // the inputs of at most 64 + 2 (bs - 1) channels' runs
+        const size_t lds = (size_t)(bs >= 64 ? ((63 / bs) + 2) * bs : 64 + 2 * bs) * sizeof(float);
+        if (lds <= 64 * 1024) {
+            hipLaunchKernelGGL(block_gates_rows_kernel, dim3(tokens, (width + 63) / 64), dim3(256), lds, stream, a_out, b_out, u,
+                               width, bs, wa, wi, w_dtype, ba, bi, rate);
+            KVA_CHECK_LAUNCH("block_gates");
+            return KVA_OK;
+        }
+    }
+    KVA_REQUIRE(blocks <= 65535 && (tokens + BG_BM - 1) / BG_BM <= 65535, "block_gates: too many runs or tokens for one launch");
+    hipLaunchKernelGGL(block_gates_kernel, dim3((bs + BG_BN - 1) / BG_BN, blocks, (tokens + BG_BM - 1) / BG_BM), dim3(256), 0, stream, a_out, b_out,
                        u, tokens, width, bs, wa, wi, w_dtype, ba, bi, rate);
     KVA_CHECK_LAUNCH("block_gates");
     return KVA_OK;
@@ -1010,6 +1104,93 @@ matrix_memory_kernel(float *__restrict__ out, float *__restrict__ state, size_t 
     if (lane == 0) *m_g = m;
 }
 
+// The same for key sizes up to 128, with the state in registers: a workgroup of four wavefronts takes the 16
+// value columns, a wavefront four of them, 16 lanes a column; lane = 16 c + r owns rows r, r + 16, ... of its
+// column of S and of its copy of n (RP of each), sums over the rows are rotations inside a row of lanes, and
+// the four wavefronts share the staged tokens (32 at a time).
+#define MM_REG_STAGE 32
+template <int RP>
+__global__ void __launch_bounds__(256)
+matrix_memory_reg_kernel(float *__restrict__ out, float *__restrict__ state, size_t seat_stride, int state_off,
+                         const void *__restrict__ y, int y_dtype, int y_stride, int q_off, int k_off, int v_off,
+                         const float *__restrict__ gates, float cap, float q_mul, const int *__restrict__ entry_q_start,
+                         const int *__restrict__ entry_seat, int heads, int dim, int vdim) {
+    extern __shared__ float lds[];
+    const int e = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * REC_COLS;
+    const int q0 = entry_q_start[e], n = entry_q_start[e + 1] - q0;
+    if (n <= 0) return;
+    const int lane = threadIdx.x % KVA_WAVE, wave = threadIdx.x / KVA_WAVE;
+    const int r16 = lane % 16, cw = 4 * wave + lane / 16, col = col0 + cw;
+    const bool col_on = col < vdim;
+    const int dpad = 16 * RP;
+    float *qs = lds;                                   // [MM_REG_STAGE][dpad]
+    float *ks = qs + MM_REG_STAGE * dpad;              // [MM_REG_STAGE][dpad]
+    float *vs = ks + MM_REG_STAGE * dpad;              // [MM_REG_STAGE][16]
+    float *gs = vs + MM_REG_STAGE * REC_COLS;          // [MM_REG_STAGE][2]
+    float *row = state + (size_t)entry_seat[e] * seat_stride + state_off;
+    float *S_g = row + (size_t)h * dim * vdim;
+    const int tiles = gridDim.x, tile = blockIdx.x;
+    float *n_g = row + (size_t)heads * dim * vdim + ((size_t)h * tiles + tile) * dim;
+    float *m_g = row + (size_t)heads * dim * vdim + (size_t)heads * tiles * dim + (size_t)h * tiles + tile;
+    float S[RP], N[RP];
+#pragma unroll
+    for (int i = 0; i < RP; ++i) {
+        const int r = r16 + 16 * i;
+        S[i] = (r < dim && col_on) ? S_g[(size_t)r * vdim + col] : 0.f;
+        N[i] = r < dim ? n_g[r] : 0.f;
+    }
+    float m = *m_g;
+    for (int t0 = 0; t0 < n; t0 += MM_REG_STAGE) {
+        const int cnt = min(MM_REG_STAGE, n - t0);
+        __syncthreads();
+        for (int i = threadIdx.x; i < cnt * dpad; i += blockDim.x) {
+            const int tt = i / dpad, r = i % dpad;
+            const size_t at = (size_t)(q0 + t0 + tt) * y_stride;
+            qs[i] = r < dim ? rec_ld(y, y_dtype, at + q_off + h * dim + r) * q_mul : 0.f;
+            ks[i] = r < dim ? rec_ld(y, y_dtype, at + k_off + h * dim + r) : 0.f;
+        }
+        for (int i = threadIdx.x; i < cnt * REC_COLS; i += blockDim.x) {
+            const int tt = i / REC_COLS, cc = i % REC_COLS;
+            vs[i] = col0 + cc < vdim ? rec_ld(y, y_dtype, (size_t)(q0 + t0 + tt) * y_stride + v_off + h * vdim + col0 + cc) : 0.f;
+        }
+        if (threadIdx.x < cnt) {
+            const float zi = gates[(size_t)(q0 + t0 + threadIdx.x) * 2 * heads + h];
+            const float zf = gates[(size_t)(q0 + t0 + threadIdx.x) * 2 * heads + heads + h];
+            const float f = cap * tanhf(zf / cap);
+            gs[2 * threadIdx.x] = cap * tanhf(zi / cap);
+            gs[2 * threadIdx.x + 1] = -rec_softplus(-f);
+        }
+        __syncthreads();
+        for (int tt = 0; tt < cnt; ++tt) {
+            const float gi = gs[2 * tt], gf = gs[2 * tt + 1];
+            const float m_new = fmaxf(gf + m, gi);
+            const float keep = expf(gf + m - m_new), take = expf(gi - m_new);
+            m = m_new;
+            const float tv = take * vs[tt * REC_COLS + cw];
+            float num = 0.f, nq = 0.f;
+#pragma unroll
+            for (int i = 0; i < RP; ++i) {
+                const float kv = ks[tt * dpad + r16 + 16 * i], qv = qs[tt * dpad + r16 + 16 * i];
+                S[i] = keep * S[i] + kv * tv;
+                N[i] = keep * N[i] + take * kv;
+                num += S[i] * qv;
+                nq += N[i] * qv;
+            }
+            num = row16_sum(num);
+            nq = row16_sum(nq);
+            if (r16 == 0 && col_on)
+                out[(size_t)(q0 + t0 + tt) * heads * vdim + (size_t)h * vdim + col] = num / (fmaxf(fabsf(nq), expf(-m)) + 1e-6f);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < RP; ++i) {
+        const int r = r16 + 16 * i;
+        if (r < dim && col_on) S_g[(size_t)r * vdim + col] = S[i];
+        if (r < dim && cw == 0) n_g[r] = N[i];
+    }
+    if (threadIdx.x == 0) *m_g = m;
+}
+
 extern "C" int kva_matrix_memory_state(int heads, int dim, int vdim) {
     const int tiles = (vdim + REC_COLS - 1) / REC_COLS;
     return heads * dim * vdim + heads * tiles * (dim + 1);
@@ -1023,6 +1204,23 @@ extern "C" int kva_matrix_memory(float *out, float *state, long long seat_stride
     KVA_REQUIRE(heads > 0 && dim > 0 && dim <= REC_MAX_DIM && vdim > 0 && cap > 0.f, "matrix_memory: bad sizes (key size up to %d)", REC_MAX_DIM);
     KVA_REQUIRE(entries >= 0 && entries <= 65535 && heads <= 65535, "matrix_memory: bad batch");
     if (entries == 0) return KVA_OK;
+    const dim3 grid((vdim + REC_COLS - 1) / REC_COLS, heads, entries);
+    if (dim <= 128) {
+        // (which kernel runs depends on the key size alone: a token's numbers are the same in any batch)
+        const int rp = dim <= 16 ? 1 : dim <= 32 ? 2 : dim <= 64 ? 4 : 8;
+        const size_t reg_lds = ((size_t)2 * MM_REG_STAGE * 16 * rp + MM_REG_STAGE * REC_COLS + 2 * MM_REG_STAGE) * sizeof(float);
+#define KVA_MM_REG(RP)                                                                                                      \
+    hipLaunchKernelGGL(matrix_memory_reg_kernel<RP>, grid, dim3(256), reg_lds, stream, out, state, (size_t)seat_stride,     \
+                       state_off, y, y_dtype, y_stride, q_off, k_off, v_off, gates, cap, q_mul, entry_q_start, entry_seat,  \
+                       heads, dim, vdim)
+        if (rp == 1) KVA_MM_REG(1);
+        else if (rp == 2) KVA_MM_REG(2);
+        else if (rp == 4) KVA_MM_REG(4);
+        else KVA_MM_REG(8);
+#undef KVA_MM_REG
+        KVA_CHECK_LAUNCH("matrix_memory");
+        return KVA_OK;
+    }
     const size_t lds = ((size_t)2 * dim * REC_COLS + (size_t)2 * MM_STAGE * dim + MM_STAGE * REC_COLS + 2 * MM_STAGE) * sizeof(float);
     KVA_REQUIRE(lds <= 160 * 1024, "matrix_memory: a key size of %d does not fit the local memory", dim);
     if (lds > 64 * 1024)

@@ -432,6 +432,136 @@ hyper_step_kernel(float *__restrict__ x, const void *__restrict__ y, int y_dtype
                       (row_s[j] - mean) * inv * ld_as_float(nw, w_dtype, j) + (nb ? ld_as_float(nb, w_dtype, j) : 0.f));
 }
 
+// The same with a row's elements in registers (a width that is a multiple of 4 up to 1,024 * ITERS, fp32 or
+// bf16 operands): a thread takes 4 neighbouring columns ITERS times, asks for all its loads - the S copies,
+// the branch output, the norm's weight and bias - before it uses any, and rows move 16 bytes a lane.  At a
+// few rows the launch is as long as its chain of trips to memory; this makes it one trip.
+__device__ inline void hyper_ld4(const void *p, int dtype, size_t i, float (&f)[4]) {
+    if (dtype == KVA_F32) {
+        const float4 v = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(p) + i);
+        f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+    } else {
+        const uint2 v = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(p) + i);
+        f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+        f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+    }
+}
+
+template <int S, int ITERS>
+__global__ void __launch_bounds__(256)
+hyper_step_vec_kernel(float *__restrict__ x, const void *__restrict__ y, int y_dtype, const float *__restrict__ mix,
+                      const float *__restrict__ out_w, float mult, const float *__restrict__ in_w,
+                      const void *__restrict__ nw, const void *__restrict__ nb, int w_dtype, float eps,
+                      void *__restrict__ out, int out_dtype, const int *__restrict__ row_idx, int width) {
+    __shared__ float red_s[4];
+    __shared__ HyperCoefficients co;
+    const int r = blockIdx.x;
+    const size_t row = (size_t)(row_idx ? row_idx[r] : r);
+    float *xr = x + row * S * width;
+    float v[ITERS][S][4], yv[ITERS][4], wv[ITERS][4], bv[ITERS][4];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int j = (threadIdx.x + it * 256) * 4;
+        const bool on = j < width;
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+            const float4 t = on ? *reinterpret_cast<const float4 *>(xr + (size_t)s * width + j) : make_float4(0.f, 0.f, 0.f, 0.f);
+            v[it][s][0] = t.x; v[it][s][1] = t.y; v[it][s][2] = t.z; v[it][s][3] = t.w;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) yv[it][e] = wv[it][e] = bv[it][e] = 0.f;
+        if (on && y) hyper_ld4(y, y_dtype, row * width + j, yv[it]);
+        if (on && out) hyper_ld4(nw, w_dtype, j, wv[it]);
+        if (on && out && nb) hyper_ld4(nb, w_dtype, j, bv[it]);
+    }
+    if (threadIdx.x < S * S) co.mix[threadIdx.x] = y ? mix[threadIdx.x] : 0.f;
+    if (threadIdx.x < S) {
+        co.out_w[threadIdx.x] = y ? out_w[threadIdx.x] * mult : 0.f;
+        co.in_w[threadIdx.x] = out ? in_w[threadIdx.x] : 0.f;
+    }
+    __syncthreads();
+    float u[ITERS][4];
+    float sum = 0.f;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int j = (threadIdx.x + it * 256) * 4;
+        const bool on = j < width;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (y) {
+                float nv[S];
+#pragma unroll
+                for (int t = 0; t < S; ++t) {
+                    float acc = 0.f;
+#pragma unroll
+                    for (int s = 0; s < S; ++s) acc += co.mix[s * S + t] * v[it][s][e];
+                    nv[t] = acc + co.out_w[t] * yv[it][e];
+                }
+#pragma unroll
+                for (int t = 0; t < S; ++t) v[it][t][e] = nv[t];
+            }
+            float a = 0.f;
+#pragma unroll
+            for (int s = 0; s < S; ++s) a += co.in_w[s] * v[it][s][e];
+            u[it][e] = on ? a : 0.f;
+            sum += u[it][e];
+        }
+        if (y && !row_idx && on) {
+#pragma unroll
+            for (int t = 0; t < S; ++t)
+                *reinterpret_cast<float4 *>(xr + (size_t)t * width + j) = make_float4(v[it][t][0], v[it][t][1], v[it][t][2], v[it][t][3]);
+        }
+    }
+    if (!out) return;
+    const float mean = block_sum(sum, red_s, 4) / (float)width;
+    float sq = 0.f;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const bool on = (threadIdx.x + it * 256) * 4 < width;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float d = on ? u[it][e] - mean : 0.f;
+            sq += d * d;
+        }
+    }
+    const float inv = 1.0f / sqrtf(block_sum(sq, red_s, 4) / (float)width + eps);
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int j = (threadIdx.x + it * 256) * 4;
+        if (j >= width) continue;
+        float o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = (u[it][e] - mean) * inv * wv[it][e] + bv[it][e];
+        if (out_dtype == KVA_F32) {
+            *reinterpret_cast<float4 *>(reinterpret_cast<float *>(out) + (size_t)r * width + j) = make_float4(o[0], o[1], o[2], o[3]);
+        } else {
+            *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(out) + (size_t)r * width + j) =
+                make_uint2((uint32_t)float_to_bf16_bits(o[0]) | ((uint32_t)float_to_bf16_bits(o[1]) << 16),
+                           (uint32_t)float_to_bf16_bits(o[2]) | ((uint32_t)float_to_bf16_bits(o[3]) << 16));
+        }
+    }
+}
+
+template <int S>
+static bool hyper_step_vec(float *x, const void *y, int y_dtype, const float *mix, const float *out_w, float mult,
+                           const float *in_w, const void *norm_w, const void *norm_b, int w_dtype, float eps, void *out,
+                           int out_dtype, const int *row_idx, int rows, int width, hipStream_t stream) {
+    // (which kernel runs depends on sizes and types alone, never on the rows: a row's numbers are the same in any batch)
+    if (width % 4 || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(norm_w) |
+                       reinterpret_cast<uintptr_t>(norm_b) | reinterpret_cast<uintptr_t>(out)) & 15))
+        return false;
+#define KVA_HYPER_VEC(ITERS)                                                                                               \
+    hipLaunchKernelGGL((hyper_step_vec_kernel<S, ITERS>), dim3(rows), dim3(256), 0, stream, x, y, y_dtype, mix, out_w, mult,  \
+                       in_w, norm_w, norm_b, w_dtype, eps, out, out_dtype, row_idx, width)
+    if (width <= 1024) KVA_HYPER_VEC(1);
+    else if (width <= 2048 && S <= 8) KVA_HYPER_VEC(2);
+    else if (width <= 4096 && S <= 4) KVA_HYPER_VEC(4);
+    else if (width <= 8192 && S <= 2) KVA_HYPER_VEC(8);
+    else return false;
+#undef KVA_HYPER_VEC
+    return true;
+}
+
 extern "C" int kva_hyper_step(float *x, int streams, const void *y, int y_dtype, const float *mix, const float *out_w,
                               float mult, const float *in_w, const void *norm_w, const void *norm_b, int w_dtype, float eps,
                               void *out, int out_dtype, const int *row_idx, int rows, int width, hipStream_t stream) {
@@ -443,6 +573,18 @@ extern "C" int kva_hyper_step(float *x, int streams, const void *y, int y_dtype,
     KVA_REQUIRE(y || out, "hyper_step: nothing to do");
     KVA_REQUIRE(!row_idx || out, "hyper_step: rows are gathered for the read-out only");
     if (rows == 0) return KVA_OK;
+    bool done = false;
+    switch (streams) {
+        case 1: done = hyper_step_vec<1>(x, y, y_dtype, mix, out_w, mult, in_w, norm_w, norm_b, w_dtype, eps, out, out_dtype, row_idx, rows, width, stream); break;
+        case 2: done = hyper_step_vec<2>(x, y, y_dtype, mix, out_w, mult, in_w, norm_w, norm_b, w_dtype, eps, out, out_dtype, row_idx, rows, width, stream); break;
+        case 3: done = hyper_step_vec<3>(x, y, y_dtype, mix, out_w, mult, in_w, norm_w, norm_b, w_dtype, eps, out, out_dtype, row_idx, rows, width, stream); break;
+        case 4: done = hyper_step_vec<4>(x, y, y_dtype, mix, out_w, mult, in_w, norm_w, norm_b, w_dtype, eps, out, out_dtype, row_idx, rows, width, stream); break;
+        default: break;
+    }
+    if (done) {
+        KVA_CHECK_LAUNCH("hyper_step");
+        return KVA_OK;
+    }
     const size_t lds = (size_t)width * sizeof(float);
 #define KVA_HYPER_CASE(S)                                                                                               \
     case S:                                                                                                             \

@@ -1843,6 +1843,8 @@ KERNEL_CLASSES = {
     "moe_route": "routed experts", "moe_align": "routed experts", "moe_expert_rows": "routed experts",
     "moe_combine": "routed experts", "small_product_f32": "small fp32 products",
     "norm_into_stream": "norm", "table_gate": "elementwise",
+    "hyper_step": "norm", "hyper_fill": "embedding", "bias_act": "activation",
+    "block_gates": "recurrent mixers", "linear_scan_gate": "recurrent mixers", "matrix_memory": "recurrent mixers",
 }
 
 
