@@ -150,7 +150,7 @@ def bonusun_config(layers: int, vocab: int, width: int = 2048) -> dict:
         {"type": "rglru", "mlp": mlp, "mixer": {"width": W, "blocks": W // 256, "conv": 4}},
         {"type": "attention", "mlp": mlp, "mixer": dict(attn, mask={"size": 1024})},
         {"type": "parallel", "mlp": mlp, "mixer": {"left": dict(attn), "left_scale": 1.0, "right_scale": 0.5,
-                                                   "right": {"heads": W // 128, "dim": 64, "vdim": 128, "gate_cap": 15.0}}},
+                                                   "right": {"heads": W // 128, "dim": 64, "vdim": 128, "gate_cap": 12.0}}},
         {"type": "attention", "mlp": mlp, "mixer": dict(attn, mask={"size": 1024})},
     ]
     return {"architecture": "Bonusun", "vocab": vocab, "width": W, "norm": {"eps": 1e-6}, "residual_mult": 0.7, "streams": 4,

@@ -78,18 +78,18 @@ CFG_A = {"architecture": "Bonusun", "vocab": 211, "width": 96, "norm": {"eps": 0
 CFG_B = {"architecture": "Bonusun", "vocab": 157, "width": 72, "norm": {"eps": 0.1}, "residual_mult": 1.0, "layers": [
     attention_layer(attention(3, 3, 20, 20, 0.3, rot=(20, 1000.0)), moe(4, 2, 16, 1.0)),
     rglru_layer(24, 24, 1, moe(1, 1, 24, 3.0)),
-    parallel_layer(attention(2, 2, 8, 12, 0.5), (1, 8, 40, 15.0), 1.0, 1.0, dense(48)),
+    parallel_layer(attention(2, 2, 8, 12, 0.5), (1, 8, 40, 12.0), 1.0, 1.0, dense(48)),
     attention_layer(attention(2, 1, 16, 32, 0.25, rot=(4, 20.0), window=1), moe(3, 2, 16, 1.0, shared=(8, 0.7)))]}
 # C: sizes at which the bf16 engine takes its matrix-core kernels: heads of 64 and 128, four query heads a kv
 #    head, values of 32 beside keys of 64, windows of 32 and 100 positions, experts over a width of 256, ONE
 #    copy of the stream with stored hyper-connection weights, a loop over the whole model.
-CFG_C = {"architecture": "Bonusun", "vocab": 257, "width": 256, "norm": {"eps": 0.02}, "residual_mult": 0.7, "streams": 1,
+CFG_C = {"architecture": "Bonusun", "vocab": 257, "width": 256, "norm": {"eps": 0.02}, "residual_mult": 0.8, "streams": 1,
          "loop": {"start": 0, "stop": 4, "times": 2}, "layers": [
-             attention_layer(attention(8, 2, 64, 64, 0.11, rot=(64, 250000.0), window=32),
-                             moe(8, 3, 64, 1.0, groups=(4, 2), scale=1.5, shared=(128, 1.5))),
-             rglru_layer(128, 2, 3, dense(384)),
-             parallel_layer(attention(4, 1, 64, 32, 0.125, rot=(32, 10000.0), factor=2.0), (4, 32, 48, 15.0), 0.8, 1.1,
-                            moe(12, 4, 64, 1.0, groups=(4, 3), scale=1.5, shared=(128, 1.5))),
+             attention_layer(attention(8, 2, 64, 64, 0.11, rot=(64, 100000.0), window=32),
+                             moe(8, 3, 64, 0.9, groups=(4, 2), scale=1.2, shared=(96, 2.0))),
+             rglru_layer(192, 3, 4, dense(320)),
+             parallel_layer(attention(4, 1, 64, 32, 0.125, rot=(32, 10000.0), factor=3.0), (2, 64, 32, 10.0), 0.9, 1.2,
+                            moe(10, 3, 96, 1.3, groups=(5, 3), scale=2.0, shared=(64, 0.9))),
              attention_layer(attention(2, 1, 128, 128, 0.09, rot=(64, 5000.0), window=100), moe(6, 2, 128, 1.2, groups=(2, 1)))]}
 # D: no layer keeps keys and values (the cache manager has no paged group): recurrences only, over two copies
 #    of the stream; seventeen taps; a run of channels wider than 64.

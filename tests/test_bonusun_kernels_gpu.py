@@ -105,7 +105,7 @@ def plain_route(logits, corr, top, groups, keep, scale, eps=1e-20):
     return torch.tensor(idx), torch.stack(wgt)
 
 
-@pytest.mark.parametrize("E, top, groups, keep", [(12, 4, 4, 3), (6, 2, 3, 2), (4, 1, 4, 2), (8, 8, 1, 1), (64, 6, 8, 2),
+@pytest.mark.parametrize("E, top, groups, keep", [(12, 3, 4, 2), (6, 2, 3, 2), (4, 1, 4, 2), (8, 8, 1, 1), (64, 6, 8, 2),
                                                   (130, 5, 1, 1), (9, 3, 3, 1), (16, 4, 2, 2)])
 def test_the_router_chooses_inside_the_best_groups(E, top, groups, keep, gpu):
     T = 50
@@ -114,8 +114,8 @@ def test_the_router_chooses_inside_the_best_groups(E, top, groups, keep, gpu):
     idx = torch.empty((T, top), dtype=torch.int32, device=DEV)
     wgt = torch.empty((T, top), dtype=torch.float32, device=DEV)
     K.moe_route(logits, corr, top, idx, wgt, renormalise=True, scores="sigmoid", groups=groups, keep_groups=keep,
-                group_top=2, weight_scale=1.5, sum_eps=1e-20)
-    want_idx, want_w = plain_route(logits.cpu(), corr.cpu(), top, groups, keep, 1.5)
+                group_top=2, weight_scale=1.3, sum_eps=1e-20)
+    want_idx, want_w = plain_route(logits.cpu(), corr.cpu(), top, groups, keep, 1.3)
     assert torch.equal(idx.cpu().long(), want_idx)
     close(wgt, want_w, 1e-6)
 
@@ -231,7 +231,7 @@ def test_real_gated_recurrence_over_steps_and_seats_used_again(width, blocks, wd
         close(state[seats[r], 11:], S, 2e-5, f"state of request {r}")
 
 
-@pytest.mark.parametrize("H, d, dv", [(3, 16, 24), (1, 8, 40), (4, 32, 48), (2, 160, 8), (2, 64, 64)])
+@pytest.mark.parametrize("H, d, dv", [(3, 16, 24), (1, 8, 40), (4, 32, 40), (2, 160, 8), (2, 64, 64)])
 @pytest.mark.parametrize("ydtype", [torch.float32, torch.bfloat16])
 def test_matrix_memory_over_steps_and_seats_used_again(H, d, dv, ydtype, gpu):
     lengths, cap = [70, 2, 33], 5.0
@@ -277,7 +277,7 @@ def test_matrix_memory_over_steps_and_seats_used_again(H, d, dv, ydtype, gpu):
         close(state[seats[r], 4:4 + H * d * dv], S.reshape(-1), 5e-5, f"matrix of request {r}")
 
 
-@pytest.mark.parametrize("heads, dv", [(4, 48), (1, 40), (3, 8)])
+@pytest.mark.parametrize("heads, dv", [(4, 40), (1, 56), (3, 8)])
 def test_head_norm_with_a_weight_of_all_heads_size_and_without_a_gate(heads, dv, gpu):
     T = 5
     x, w, gate = rnd((T, heads * dv), 1), rnd((heads * dv,), 2, 0.3, 1.0), rnd((T, heads * dv + 4), 3)

@@ -23,7 +23,7 @@ def random_config(seed: int) -> dict:
             return None
         if r < 0.3:
             return U.dense(pick(48, 100, 256))
-        experts, groups = pick((1, None), (2, None), (3, None), (4, (2, 1)), (6, (3, 2)), (8, (4, 2)), (8, (8, 3)), (12, (4, 3)),
+        experts, groups = pick((1, None), (2, None), (3, None), (4, (2, 1)), (6, (3, 2)), (8, (4, 2)), (8, (8, 3)), (12, (3, 2)),
                                (16, (2, 2)), (9, (3, 3)), (5, None))
         per = experts if groups is None else experts // groups[0] * groups[1]
         top = int(rng.integers(1, min(per, 6) + 1))
@@ -32,9 +32,9 @@ def random_config(seed: int) -> dict:
 
     def attention():
         kv, dim = pick(1, 2, 3), pick(8, 16, 20, 32, 48, 64, 128)
-        rot = pick(None, (dim, 10000.0), (dim // 4 * 2, 250000.0), (4, 50.0))
+        rot = pick(None, (dim, 10000.0), (dim // 4 * 2, 300000.0), (4, 50.0))
         return U.attention(kv * pick(1, 2, 4), kv, dim, pick(dim, 8, 16, 32, 80), pick(0.1, 0.125, 0.3), rot=rot,
-                           window=pick(None, None, 1, 5, 16, 33, 96), factor=pick(None, 2.0, 8.0) if rot else None)
+                           window=pick(None, None, 1, 5, 16, 33, 80), factor=pick(None, 2.0, 8.0) if rot else None)
 
     layers = []
     for i in range(int(rng.integers(2, 6))):
@@ -42,7 +42,7 @@ def random_config(seed: int) -> dict:
         if kind == "attention":
             layers.append(U.attention_layer(attention(), mlp()))
         elif kind == "parallel":
-            right = (pick(1, 2, 4), pick(8, 16, 32, 40, 64, 136), pick(8, 24, 48, 64), float(pick(3.0, 5.0, 15.0)))
+            right = (pick(1, 2, 4), pick(8, 16, 32, 40, 64, 136), pick(8, 24, 48, 64), float(pick(3.0, 5.0, 12.0)))
             layers.append(U.parallel_layer(attention(), right, pick(0.5, 1.0, 1.2), pick(0.5, 1.0, 1.7), mlp()))
         else:
             blocks = pick(1, 2, 4, 8)
