@@ -96,7 +96,16 @@ CFG_C = {"architecture": "Bonusun", "vocab": 257, "width": 256, "norm": {"eps": 
 CFG_D = {"architecture": "Bonusun", "vocab": 131, "width": 64, "norm": {"eps": 0.05}, "residual_mult": 1.3, "streams": 2,
          "layers": [rglru_layer(160, 2, 17, moe(2, 1, 32, 1.0, shared=(32, 1.0))), rglru_layer(32, 4, 3),
                     rglru_layer(64, 1, 2, dense(96))]}
-CONFIGS = {"A": (CFG_A, 5), "B": (CFG_B, 6), "C": (CFG_C, 7), "D": (CFG_D, 8)}
+# E: a width of 512, where one or two decoded tokens take the matrix-vector kernels; heads of 128 with values of
+#    64; five copies of the stream (more than the kernel that keeps a row in registers takes); a vocabulary
+#    that is no multiple of 8; a memory with keys of 136 channels (its state in LDS).
+CFG_E = {"architecture": "Bonusun", "vocab": 1003, "width": 512, "norm": {"eps": 0.03}, "residual_mult": 0.9, "streams": 5,
+         "layers": [
+             parallel_layer(attention(4, 2, 128, 64, 0.08, rot=(96, 40000.0), window=40), (2, 136, 24, 8.0), 1.1, 0.6,
+                            moe(16, 2, 128, 1.1, groups=(8, 4), scale=1.4, shared=(192, 1.0))),
+             rglru_layer(384, 6, 4, dense(768)),
+             attention_layer(attention(8, 8, 32, 48, 0.17, rot=(32, 1000.0), factor=1.25), moe(3, 1, 256, 2.5))]}
+CONFIGS = {"A": (CFG_A, 5), "B": (CFG_B, 6), "C": (CFG_C, 7), "D": (CFG_D, 8), "E": (CFG_E, 9)}
 
 
 def write_model(folder: str, cfg: dict, seed: int, gain: float = 1.0, edit=None) -> Tuple[str, Dict[str, torch.Tensor]]:

@@ -34,7 +34,7 @@ def engine_for(folder, dtype, **kw):
     return Engine(folder, EngineOptions(**opts))
 
 
-REQUESTS = {"A": [1, 2, 9, 40, 77], "B": [3, 33, 70], "C": [1, 5, 47, 150], "D": [2, 35, 64]}
+REQUESTS = {"A": [1, 2, 9, 40, 77], "B": [3, 33, 70], "C": [1, 5, 47, 150], "D": [2, 35, 64], "E": [2, 44, 101]}
 
 
 def requests_for(name, cfg):
@@ -49,7 +49,7 @@ def check(eng, cfg, state, reqs, steps, dtype, what, close_call=None, tolerance=
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_whole_prompts_and_the_first_tokens(name, dtype, models, gpu):
     cfg, folder, state = models[name]
     reqs = requests_for(name, cfg)
@@ -60,7 +60,7 @@ def test_whole_prompts_and_the_first_tokens(name, dtype, models, gpu):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_prefill_against_token_by_token_decoding(name, dtype, models, gpu):
     """Most of a request in one step, the rest one token at a time (windows pass over decoded tokens; the
     states, the running maxima and the convolutions' last inputs are carried from step to step); and a
@@ -84,7 +84,7 @@ def test_portions_of_any_size(name, sizes, dtype, models, gpu):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name, seed", [("A", 0), ("B", 1), ("B", 2), ("C", 3), ("C", 4), ("D", 5)])
+@pytest.mark.parametrize("name, seed", [("A", 0), ("B", 1), ("B", 2), ("C", 3), ("C", 4), ("D", 5), ("E", 6)])
 def test_mixed_batches_on_a_small_pool_reuse_pages_and_seats(name, seed, dtype, models, gpu):
     cfg, folder, state = models[name]
     lengths = [40, 3, 90, 25, 61, 2, 130, 47, 33]
@@ -223,7 +223,7 @@ def test_greedy_generation_through_the_entry_point(name, dtype, models, gpu):
     assert llm.engine.cache.free_seats == 3
 
 
-@pytest.mark.parametrize("name", ["A", "C"])
+@pytest.mark.parametrize("name", ["A", "C", "E"])
 def test_decode_steps_from_graphs_equal_eager_steps(name, models, gpu):
     """A bf16 decode step replayed from its HIP graph gives bit for bit what the eager step gives (the copies
     of the stream, states, convolution inputs and routed experts included), replay after replay."""
