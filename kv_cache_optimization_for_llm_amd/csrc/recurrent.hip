@@ -1126,7 +1126,7 @@ matrix_memory_reg_kernel(float *__restrict__ out, float *__restrict__ state, siz
     float *qs = lds;                                   // [MM_REG_STAGE][dpad]
     float *ks = qs + MM_REG_STAGE * dpad;              // [MM_REG_STAGE][dpad]
     float *vs = ks + MM_REG_STAGE * dpad;              // [MM_REG_STAGE][16]
-    float *gs = vs + MM_REG_STAGE * REC_COLS;          // [MM_REG_STAGE][2]
+    float *gs = vs + MM_REG_STAGE * REC_COLS;          // [MM_REG_STAGE][3]: e^(f + m - m'), e^(i - m'), e^(-m') of every token
     float *row = state + (size_t)entry_seat[e] * seat_stride + state_off;
     float *S_g = row + (size_t)h * dim * vdim;
     const int tiles = gridDim.x, tile = blockIdx.x;
@@ -1140,32 +1140,79 @@ matrix_memory_reg_kernel(float *__restrict__ out, float *__restrict__ state, siz
         N[i] = r < dim ? n_g[r] : 0.f;
     }
     float m = *m_g;
+    // What a thread stages of a chunk of tokens: 2 RP elements of q and of k, 2 of v, and - the first wavefront's
+    // lanes - a token's two gate inputs.  All of it is asked for before any of it is used, and the next chunk's
+    // while this one's tokens are walked.
+    constexpr int PER = MM_REG_STAGE * 16 * RP / 256;
+    float pq[PER], pk[PER], pv[2], pzi = 0.f, pzf = 0.f;
+    auto fetch = [&](int t0) {
+        const int cnt = min(MM_REG_STAGE, n - t0);
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int i = threadIdx.x + j * 256, tt = i / dpad, r = i % dpad;
+            const bool in = tt < cnt && r < dim;
+            const size_t at = (size_t)(q0 + t0 + (in ? tt : 0)) * y_stride + h * dim + (in ? r : 0);
+            pq[j] = in ? rec_ld(y, y_dtype, at + q_off) * q_mul : 0.f;
+            pk[j] = in ? rec_ld(y, y_dtype, at + k_off) : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int i = threadIdx.x + j * 256, tt = i / REC_COLS, cc = i % REC_COLS;
+            const bool in = tt < cnt && col0 + cc < vdim;
+            pv[j] = in ? rec_ld(y, y_dtype, (size_t)(q0 + t0 + tt) * y_stride + v_off + h * vdim + col0 + cc) : 0.f;
+        }
+        if (threadIdx.x < cnt) {
+            pzi = gates[(size_t)(q0 + t0 + threadIdx.x) * 2 * heads + h];
+            pzf = gates[(size_t)(q0 + t0 + threadIdx.x) * 2 * heads + heads + h];
+        }
+    };
+    fetch(0);
     for (int t0 = 0; t0 < n; t0 += MM_REG_STAGE) {
         const int cnt = min(MM_REG_STAGE, n - t0);
         __syncthreads();
-        for (int i = threadIdx.x; i < cnt * dpad; i += blockDim.x) {
-            const int tt = i / dpad, r = i % dpad;
-            const size_t at = (size_t)(q0 + t0 + tt) * y_stride;
-            qs[i] = r < dim ? rec_ld(y, y_dtype, at + q_off + h * dim + r) * q_mul : 0.f;
-            ks[i] = r < dim ? rec_ld(y, y_dtype, at + k_off + h * dim + r) : 0.f;
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            qs[threadIdx.x + j * 256] = pq[j];
+            ks[threadIdx.x + j * 256] = pk[j];
         }
-        for (int i = threadIdx.x; i < cnt * REC_COLS; i += blockDim.x) {
-            const int tt = i / REC_COLS, cc = i % REC_COLS;
-            vs[i] = col0 + cc < vdim ? rec_ld(y, y_dtype, (size_t)(q0 + t0 + tt) * y_stride + v_off + h * vdim + col0 + cc) : 0.f;
-        }
-        if (threadIdx.x < cnt) {
-            const float zi = gates[(size_t)(q0 + t0 + threadIdx.x) * 2 * heads + h];
-            const float zf = gates[(size_t)(q0 + t0 + threadIdx.x) * 2 * heads + heads + h];
-            const float f = cap * tanhf(zf / cap);
-            gs[2 * threadIdx.x] = cap * tanhf(zi / cap);
-            gs[2 * threadIdx.x + 1] = -rec_softplus(-f);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) vs[threadIdx.x + j * 256] = pv[j];
+        if (wave == 0) {
+            // The running maxima of the staged tokens, by the first wavefront, lane = token: with F_t the sum of
+            // the log forget gates up to t, m_t = F_t + max(m, max_(j <= t) (i_j - F_j)) - a prefix sum and a
+            // prefix maximum over the lanes instead of a walk - and from them what the walk below multiplies by.
+            const bool on = lane < cnt;
+            float gi = -INFINITY, gf = 0.f;
+            if (on) {
+                gi = cap * tanhf(pzi / cap);
+                gf = -rec_softplus(-cap * tanhf(pzf / cap));
+            }
+            float F = gf;
+#pragma unroll
+            for (int o = 1; o < MM_REG_STAGE; o <<= 1) {
+                const float up = __shfl_up(F, o, KVA_WAVE);
+                if (lane >= o) F += up;
+            }
+            float A = gi - F;
+#pragma unroll
+            for (int o = 1; o < MM_REG_STAGE; o <<= 1) {
+                const float up = __shfl_up(A, o, KVA_WAVE);
+                if (lane >= o) A = fmaxf(A, up);
+            }
+            const float mt = F + fmaxf(m, A);
+            float prev = __shfl_up(mt, 1, KVA_WAVE);
+            if (lane == 0) prev = m;
+            if (on) {
+                gs[3 * lane] = expf(gf + prev - mt);
+                gs[3 * lane + 1] = expf(gi - mt);
+                gs[3 * lane + 2] = expf(-mt);
+            }
+            m = __shfl(mt, cnt - 1, KVA_WAVE);
         }
         __syncthreads();
+        if (t0 + MM_REG_STAGE < n) fetch(t0 + MM_REG_STAGE);
         for (int tt = 0; tt < cnt; ++tt) {
-            const float gi = gs[2 * tt], gf = gs[2 * tt + 1];
-            const float m_new = fmaxf(gf + m, gi);
-            const float keep = expf(gf + m - m_new), take = expf(gi - m_new);
-            m = m_new;
+            const float keep = gs[3 * tt], take = gs[3 * tt + 1], floor_den = gs[3 * tt + 2];
             const float tv = take * vs[tt * REC_COLS + cw];
             float num = 0.f, nq = 0.f;
 #pragma unroll
@@ -1179,7 +1226,7 @@ matrix_memory_reg_kernel(float *__restrict__ out, float *__restrict__ state, siz
             num = row16_sum(num);
             nq = row16_sum(nq);
             if (r16 == 0 && col_on)
-                out[(size_t)(q0 + t0 + tt) * heads * vdim + (size_t)h * vdim + col] = num / (fmaxf(fabsf(nq), expf(-m)) + 1e-6f);
+                out[(size_t)(q0 + t0 + tt) * heads * vdim + (size_t)h * vdim + col] = num / (fmaxf(fabsf(nq), floor_den) + 1e-6f);
         }
     }
 #pragma unroll
@@ -1208,7 +1255,7 @@ extern "C" int kva_matrix_memory(float *out, float *state, long long seat_stride
     if (dim <= 128) {
         // (which kernel runs depends on the key size alone: a token's numbers are the same in any batch)
         const int rp = dim <= 16 ? 1 : dim <= 32 ? 2 : dim <= 64 ? 4 : 8;
-        const size_t reg_lds = ((size_t)2 * MM_REG_STAGE * 16 * rp + MM_REG_STAGE * REC_COLS + 2 * MM_REG_STAGE) * sizeof(float);
+        const size_t reg_lds = ((size_t)2 * MM_REG_STAGE * 16 * rp + MM_REG_STAGE * REC_COLS + 3 * MM_REG_STAGE) * sizeof(float);
 #define KVA_MM_REG(RP)                                                                                                      \
     hipLaunchKernelGGL(matrix_memory_reg_kernel<RP>, grid, dim3(256), reg_lds, stream, out, state, (size_t)seat_stride,     \
                        state_off, y, y_dtype, y_stride, q_off, k_off, v_off, gates, cap, q_mul, entry_q_start, entry_seat,  \
