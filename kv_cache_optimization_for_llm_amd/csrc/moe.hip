@@ -37,7 +37,7 @@ __global__ void __launch_bounds__(256)
 moe_route_kernel(int *__restrict__ idx, float *__restrict__ wgt, const float *__restrict__ logits,
                  const float *__restrict__ correction, int tokens, int outputs, int top, int renormalise,
                  int over_chosen, int sigmoid_scores, int groups, int keep_groups, int group_top, float weight_scale,
-                 float sum_eps) {
+                 float sum_eps, int logits_stride) {
     __shared__ float choice_s[4][KVA_WAVE * MOE_ROUTE_PER_LANE];
     const int lane = threadIdx.x % KVA_WAVE;
     const int t = blockIdx.x * (blockDim.x / KVA_WAVE) + threadIdx.x / KVA_WAVE;
@@ -48,7 +48,7 @@ moe_route_kernel(int *__restrict__ idx, float *__restrict__ wgt, const float *__
 #pragma unroll
     for (int j = 0; j < MOE_ROUTE_PER_LANE; ++j) {
         const int e = lane + j * KVA_WAVE;
-        s[j] = e < outputs ? logits[(size_t)t * outputs + e] : -INFINITY;
+        s[j] = e < outputs ? logits[(size_t)t * logits_stride + e] : -INFINITY;
         mx = fmaxf(mx, s[j]);
     }
     mx = wave_max(mx);
@@ -66,10 +66,10 @@ moe_route_kernel(int *__restrict__ idx, float *__restrict__ wgt, const float *__
         if (over_chosen) {
             // the logits themselves are compared, and the weights are a softmax over the chosen ones
             // alone: exp(logit - max) here, divided by the chosen ones' sum below
-            ch[j] = e < outputs ? logits[(size_t)t * outputs + e] + (correction ? correction[e] : 0.f) : -INFINITY;
+            ch[j] = e < outputs ? logits[(size_t)t * logits_stride + e] + (correction ? correction[e] : 0.f) : -INFINITY;
         } else {
             // scores: the softmax over all outputs, or every output's own sigmoid
-            s[j] = sigmoid_scores ? (e < outputs ? 1.f / (1.f + expf(-logits[(size_t)t * outputs + e])) : 0.f) : s[j] / sum;
+            s[j] = sigmoid_scores ? (e < outputs ? 1.f / (1.f + expf(-logits[(size_t)t * logits_stride + e])) : 0.f) : s[j] / sum;
             ch[j] = e < outputs ? s[j] + (correction ? correction[e] : 0.f) : -INFINITY;
         }
     }
@@ -153,7 +153,10 @@ moe_route_kernel(int *__restrict__ idx, float *__restrict__ wgt, const float *__
 
 extern "C" int kva_moe_route(int *idx, float *wgt, const float *logits, const float *correction, int tokens,
                              int outputs, int top, int renormalise, int over_chosen, int sigmoid_scores, int groups,
-                             int keep_groups, int group_top, float weight_scale, float sum_eps, hipStream_t stream) {
+                             int keep_groups, int group_top, float weight_scale, float sum_eps, int logits_stride,
+                             hipStream_t stream) {
+    // logits_stride: elements between two tokens' rows of logits (the logits may be the first columns of a wider product)
+    KVA_REQUIRE(logits_stride >= outputs, "moe_route: a row of logits holds at least the %d outputs", outputs);
     KVA_REQUIRE(groups >= 1 && groups <= KVA_WAVE && outputs % groups == 0 && keep_groups >= 1 && keep_groups <= groups &&
                     group_top >= 1,
                 "moe_route: %d groups (at most %d, dividing the %d outputs) of which %d are kept", groups, KVA_WAVE, outputs,
@@ -168,7 +171,7 @@ extern "C" int kva_moe_route(int *idx, float *wgt, const float *logits, const fl
     if (tokens == 0) return KVA_OK;
     hipLaunchKernelGGL(moe_route_kernel, dim3((tokens + 3) / 4), dim3(256), 0, stream, idx, wgt, logits, correction,
                        tokens, outputs, top, renormalise, over_chosen, sigmoid_scores, groups, keep_groups, group_top,
-                       weight_scale, sum_eps);
+                       weight_scale, sum_eps, logits_stride);
     KVA_CHECK_LAUNCH("moe_route");
     return KVA_OK;
 }
@@ -434,10 +437,10 @@ __device__ inline float moe_ld(const void *p, int dtype, size_t i) {
 __global__ void __launch_bounds__(256)
 moe_combine_kernel(void *__restrict__ out, const void *__restrict__ x, int dtype, const float *__restrict__ rows,
                    const int *__restrict__ idx, const float *__restrict__ wgt, const void *__restrict__ extra,
-                   const float *__restrict__ extra_gate, int width, int top, int experts) {
+                   const float *__restrict__ extra_gate, int extra_gate_stride, int width, int top, int experts) {
     const size_t t = blockIdx.x;
-    // (optional) the addend enters times sigmoid(extra_gate[t]), one number a token
-    const float eg = extra && extra_gate ? 1.f / (1.f + expf(-extra_gate[t])) : 1.f;
+    // (optional) the addend enters times sigmoid(extra_gate[t * stride]), one number a token (a column of a wider array)
+    const float eg = extra && extra_gate ? 1.f / (1.f + expf(-extra_gate[t * extra_gate_stride])) : 1.f;
     if (width % 4 == 0 && ((reinterpret_cast<uintptr_t>(rows) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
         // four neighbouring columns a thread, 16 bytes of every row at a time; the additions per column are
         // in the order of the scalar loop below
@@ -485,13 +488,13 @@ moe_combine_kernel(void *__restrict__ out, const void *__restrict__ x, int dtype
 }
 
 extern "C" int kva_moe_combine(void *out, const void *x, int dtype, const float *rows, const int *idx,
-                               const float *wgt, const void *extra, const float *extra_gate, int tokens, int width,
-                               int top, int experts, hipStream_t stream) {
+                               const float *wgt, const void *extra, const float *extra_gate, int extra_gate_stride,
+                               int tokens, int width, int top, int experts, hipStream_t stream) {
     KVA_REQUIRE(out && x && rows && idx && wgt && width > 0 && top > 0, "moe_combine: missing operand");
     KVA_REQUIRE(dtype == KVA_BF16 || dtype == KVA_F32, "moe_combine: unsupported dtype %d", dtype);
     if (tokens <= 0) return KVA_OK;
     hipLaunchKernelGGL(moe_combine_kernel, dim3(tokens), dim3(256), 0, stream, out, x, dtype, rows, idx, wgt, extra, extra_gate,
-                       width, top, experts);
+                       extra_gate_stride, width, top, experts);
     KVA_CHECK_LAUNCH("moe_combine");
     return KVA_OK;
 }

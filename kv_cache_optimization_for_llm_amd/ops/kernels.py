@@ -1711,14 +1711,16 @@ def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int
     tokens, outputs = logits.shape
     if scores not in ("softmax", "sigmoid"):
         raise KernelError(f"moe_route: scores {scores!r} is neither 'softmax' nor 'sigmoid'")
+    if logits.dim() != 2 or logits.stride(1) != 1:
+        raise KernelError("moe_route: the logits are rows with unit stride (possibly the first columns of a wider array)")
     if logits.dtype != torch.float32 or idx.shape != (tokens, top) or wgt.shape != (tokens, top) \
             or (correction is not None and correction.shape != (outputs,)):
         raise KernelError(f"moe_route: logits {tuple(logits.shape)}, idx {tuple(idx.shape)}, wgt {tuple(wgt.shape)} do not fit")
-    check(hip_lib().kva_moe_route(_dev(idx, "idx", torch.int32), _dev(wgt, "wgt", torch.float32), _dev(logits, "logits"),
+    check(hip_lib().kva_moe_route(_dev(idx, "idx", torch.int32), _dev(wgt, "wgt", torch.float32), _dev(logits, "logits", contiguous=False),
                                   _opt(correction, "correction", torch.float32), tokens, outputs, int(top),
                                   1 if renormalise else 0, 1 if over_chosen else 0, 1 if scores == "sigmoid" else 0,
                                   int(groups), int(keep_groups), int(group_top), float(weight_scale), float(sum_eps),
-                                  _stream()), "moe_route")
+                                  logits.stride(0) if tokens > 1 else outputs, _stream()), "moe_route")
 
 
 def moe_tiles(slots: int, experts: int) -> int:
@@ -1807,9 +1809,16 @@ def moe_combine(x: torch.Tensor, rows: torch.Tensor, idx: torch.Tensor, wgt: tor
     """``out[t] = sum over the token's choices`` of the slot's row of ``rows`` (fp32 ``[T * top, width]``,
     already weighted) or, for a choice past the real ``experts`` (an identity expert), ``wgt * x[t]``;
     ``extra`` (x's shape and type: what an expert that every token uses returned) is added last - times
-    ``sigmoid(extra_gate[t])`` with ``extra_gate`` (fp32, one number a token)."""
+    ``sigmoid(extra_gate[t])`` with ``extra_gate`` (fp32, one number a token; it may be a column of a wider array)."""
     if extra_gate is not None and (extra is None or extra_gate.numel() != x.shape[0] or extra_gate.dtype != torch.float32):
         raise KernelError("moe_combine: the addend's gate is fp32, one number a token")
+    gate_stride = 1
+    if extra_gate is not None:
+        if extra_gate.dim() == 2:
+            extra_gate = extra_gate[:, 0]
+        if extra_gate.dim() != 1:
+            raise KernelError("moe_combine: the addend's gate is one column")
+        gate_stride = extra_gate.stride(0) if extra_gate.shape[0] > 1 else 1
     tokens, width = x.shape
     top = idx.shape[1]
     if out.shape != x.shape or out.dtype != x.dtype or rows.shape != (tokens * top, width) or rows.dtype != torch.float32 \
@@ -1818,7 +1827,8 @@ def moe_combine(x: torch.Tensor, rows: torch.Tensor, idx: torch.Tensor, wgt: tor
         raise KernelError(f"moe_combine: x {tuple(x.shape)}, rows {tuple(rows.shape)}, idx {tuple(idx.shape)} do not fit")
     check(hip_lib().kva_moe_combine(_dev(out, "out"), _dev(x, "x"), dtype_code(x.dtype), _dev(rows, "rows"),
                                     _dev(idx, "idx", torch.int32), _dev(wgt, "wgt", torch.float32), _opt(extra, "extra"),
-                                    _opt(extra_gate, "extra_gate"), tokens, width, top, int(experts), _stream()), "moe_combine")
+                                    None if extra_gate is None else _dev(extra_gate, "extra_gate", contiguous=False),
+                                    int(gate_stride), tokens, width, top, int(experts), _stream()), "moe_combine")
     return out
 
 

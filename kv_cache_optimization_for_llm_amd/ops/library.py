@@ -95,10 +95,10 @@ _HIP_SIGNATURES = {
     "kva_gated_delta_rule": [P, P, LL, I, P, I, P, I, I, I, I, P, P, F, P, I, P, P, I, I, I, I, I, P],
     "kva_gated_linear_attention": [P, P, LL, I, P, I, I, I, I, I, P, I, F, P, I, P, P, I, I, I, I, P],
     "kva_head_norm_gate": [P, I, I, I, P, I, P, F, P, I, I, I, I, I, I, I, F, I, P],
-    "kva_moe_route": [P, P, P, P, I, I, I, I, I, I, I, I, I, F, F, P],
+    "kva_moe_route": [P, P, P, P, I, I, I, I, I, I, I, I, I, F, F, I, P],
     "kva_moe_align": [P, P, P, I, I, I, I, P],
     "kva_moe_expert_rows": [P, I, P, P, I, P, P, P, I, I, I, I, I, I, I, F, P],
-    "kva_moe_combine": [P, P, I, P, P, P, P, P, I, I, I, I, P],
+    "kva_moe_combine": [P, P, I, P, P, P, P, P, I, I, I, I, I, P],
     "kva_small_product_f32": [P, P, I, I, P, I, I, I, I, P, F, P, I, P],
     "kva_norm_into_stream": [P, I, P, I, P, I, P, I, I, I, F, P],
     "kva_table_gate": [P, P, I, P, I, I, I, I, P, P, I, I, I, P],

@@ -119,7 +119,12 @@ class RoutedExperts(FeedForward):
         self.router_bias = tensors[n["router_bias"]].float().contiguous() if self.has_router_bias else None
         if self.shared is not None:
             self.shared.load(tensors)
+        # the shared expert's gate is one more row of the router's product: one launch makes both in 32-bit
         self.shared_gate = tensors[n["shared_gate"]].contiguous() if self.has_shared_gate else None
+        if self.shared_gate is not None:
+            self.router = torch.cat([self.router, self.shared_gate.to(self.router.dtype)], dim=0).contiguous()
+            if self.router_bias is not None:
+                self.router_bias = torch.cat([self.router_bias, self.router_bias.new_zeros(1)]).contiguous()
         if self.experts and self.gated:
             # rows 2 j and 2 j + 1 of an expert's first matrix: output j's gate row and its up row
             ups = []
@@ -140,8 +145,10 @@ class RoutedExperts(FeedForward):
 
     def forward(self, x, ctx: MixerContext, tail=None):
         T, dev = x.shape[0], x.device
-        logits = K.small_product_f32(x, self.router, torch.empty((T, self.outputs), dtype=torch.float32, device=dev),
-                                     bias=self.router_bias)
+        cols = self.router.shape[0]              # the router's outputs, and the shared expert's gate behind them
+        product = K.small_product_f32(x, self.router, torch.empty((T, cols), dtype=torch.float32, device=dev),
+                                      bias=self.router_bias)
+        logits = product[:, :self.outputs]
         idx = torch.empty((T, self.top), dtype=torch.int32, device=dev)
         wgt = torch.empty((T, self.top), dtype=torch.float32, device=dev)
         K.moe_route(logits, self.correction, self.top, idx, wgt, self.renormalise, over_chosen=self.over_chosen,
@@ -162,7 +169,6 @@ class RoutedExperts(FeedForward):
             K.moe_expert_rows(act, self.w_down, rows, sorted_slot, tile_expert, self.top, slot_weight=wgt)
         out = torch.empty_like(x)
         extra = self.shared.forward(x, ctx) if self.shared is not None else None
-        gate = None
-        if self.shared_gate is not None:        # one number a token, in 32-bit; its sigmoid is taken where the rows are added
-            gate = K.small_product_f32(x, self.shared_gate, torch.empty((T, 1), dtype=torch.float32, device=dev))
+        # one number a token, in 32-bit; its sigmoid is taken where the rows are added
+        gate = product[:, self.outputs] if self.shared_gate is not None else None
         return K.moe_combine(x, rows, idx, wgt, self.experts, out, extra=extra, extra_gate=gate)
