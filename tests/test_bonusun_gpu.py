@@ -267,3 +267,17 @@ def test_the_serving_process_serves_the_model(models, tmp_path, gpu):
     r = json.load(open(out))
     assert r["status"] == "ok" and r["sequences_done"] == 10 and r["tokens"] == 100
     assert r["count_mismatches"] == 0 and r["budget_mismatches"] == 0 and r["errors"] == []
+
+
+def test_the_sweep_command_runs_a_configuration_file_of_this_architecture(models, tmp_path, gpu):
+    import json
+    import os
+    from kv_cache_optimization_for_llm_amd.cli import sweep
+    cfg, folder, state = models["C"]
+    out = tmp_path / "sweep.jsonl"
+    assert sweep.main(["--shapes", os.path.join(folder, "config.json"), "--batches", "3", "--cache-modes", "paged",
+                       "--prompt-len", "40", "--prompt-min", "5", "--workload", "mixed", "--new-tokens", "9",
+                       "--max-seqs", "2", "--out", str(out)]) == 0
+    line, = [json.loads(l) for l in out.read_text().splitlines()]
+    assert line["requests_done"] == 3 and line["tokens_emitted"] == 27 and line["finish_reasons"] == {"length": 3}
+    assert line["pages_reused"] > 0
